@@ -34,6 +34,7 @@ class NormSpec(PartSpec):
     eps: float = 0.0
     kind: str = "rmsnorm"
     weight_name: str = "weight"  # the tensor's name below the norm's prefix
+    weight_offset: float = 0.0   # the stored tensor plus this is the weight (1: a weight stored around zero)
 
 
 @dataclass(frozen=True)
@@ -149,6 +150,9 @@ class LatentMixerSpec(PartSpec):
     up_v_name: str = "uv"
     o_name: str = "o"
     weight_suffix: str = ""
+    sinks: bool = False        # one learned number per head joins the softmax's denominator as exp(sink), unscaled
+    sink_name: str = "sink"
+    own_kv: bool = True        # False: no down projection and no norm of its own; the layer reads another stop's rows
 
 
 @dataclass(frozen=True)
@@ -178,6 +182,89 @@ class DeltaMixerSpec(PartSpec):
     dt_bias_name: str = "dt_bias"
     norm_name: str = "norm"
     weight_suffix: str = ""
+    # what some designs' rule has besides:
+    decay: str = "head"              # "channel": one decay per head and key channel (A_log stays per head, dt_bias [heads, key_dim])
+    decay_rank: Optional[int] = None  # the decay's input is W_a2 (W_a1 h) with that many features between (names a1, a2)
+    gate_rank: Optional[int] = None   # likewise the gate's, W_g2 (W_g1 h)
+    gate_activation: str = "silu"    # or "sigmoid"
+    low_rank_suffixes: Tuple[str, str] = ("1", "2")  # appended to decay_name / gate_name for the two narrow products
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec(PartSpec):
+    """A matrix memory with exponential input and forget gates (the mLSTM cell): a recurrent mixer with, per head,
+    a matrix [key_dim, value_dim], the sum of its gated keys and a running maximum of the gates' logarithms.
+    `gate_cap` c bounds both gates' inputs by c tanh(z / c); `readout_floor` is added to the read-out's
+    denominator max(|n . q|, exp(-m))."""
+
+    hidden_size: int = 0
+    num_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    gate_cap: float = 15.0
+    norm_eps: float = 1e-6
+    readout_floor: float = 1e-6
+    kind: str = "matrix_memory"
+    q_name: str = "q"
+    k_name: str = "k"
+    v_name: str = "v"
+    gate_name: str = "g"          # the output gate sigmoid(W_g h)
+    input_gate_name: str = "i"    # with a bias
+    forget_gate_name: str = "f"   # with a bias
+    o_name: str = "o"
+    norm_name: str = "norm"       # one weight per head and value feature
+    bias_suffix: str = ".b"
+    weight_suffix: str = ""
+
+
+@dataclass(frozen=True)
+class SideBySideSpec(PartSpec):
+    """Two mixers that read the same input; the result is left_scale * left + right_scale * right.  Their
+    tensors lie below `left_prefix` and `right_prefix` of the mixer's own prefix."""
+
+    left: Optional[PartSpec] = None
+    right: Optional[PartSpec] = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    left_prefix: str = "left."
+    right_prefix: str = "right."
+    kind: str = "side_by_side"
+
+
+@dataclass(frozen=True)
+class ExpertsSpec(PartSpec):
+    """A feed-forward of `num_experts` small gated experts W_down (act(W_gate h) * (W_up h)) of which a token
+    uses `top`: router scores are the softmax of W_router h over all experts (float32); the experts form
+    `groups` equal groups of neighbours, a group's score is its largest, and only experts of the `groups_kept`
+    best groups can be chosen; the chosen experts' outputs are added with their scores times `route_scale`."""
+
+    hidden_size: int = 0
+    intermediate_size: int = 0
+    num_experts: int = 0
+    top: int = 1
+    groups: int = 1
+    groups_kept: int = 1
+    route_scale: float = 1.0
+    activation: str = "silu"
+    kind: str = "experts"
+    router_name: str = "router"
+    expert_prefix: str = "e"   # expert j's tensors lie below <expert_prefix><j>.
+    gate_name: str = "gate"
+    up_name: str = "up"
+    down_name: str = "down"
+    weight_suffix: str = ""
+
+
+@dataclass(frozen=True)
+class PairEmbeddingSpec:
+    """A second embedding table added to the first, indexed by a hash of the token before and the token:
+    row (previous * mul_prev + token * mul_cur) mod buckets; a sequence's first token takes row `buckets`,
+    the table's last.  The token before a step's first is per-request state."""
+
+    name: str
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass(frozen=True)
@@ -252,6 +339,7 @@ class ModelPlan:
     logit_scale: float = 1.0                # the logits are multiplied by this ...
     logit_softcap: Optional[float] = None   # ... and then, with a cap c, become c * tanh(logits / c)
     streams: int = 1                        # copies the residual stream is kept in (blocks of arrangement "hyper")
+    pair_embedding: Optional[PairEmbeddingSpec] = None  # a hashed table of token pairs added to the embedding
     extra: Mapping[str, Any] = field(default_factory=dict)
 
     def __post_init__(self) -> None:

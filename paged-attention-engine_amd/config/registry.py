@@ -15,19 +15,26 @@ from .model_config import ConfigError, ModelPlan
 
 # name -> callable(config.json dict) -> typed config object with a .plan() method
 _ARCHITECTURES: Dict[str, Callable[[Mapping[str, Any]], Any]] = {}
+# architectures some of whose sizes stand in a tensor's shape: their reader also takes {tensor name: shape}
+_READS_SHAPES = set()
 
 
-def register_architecture(name: str, config_reader: Callable[[Mapping[str, Any]], Any]) -> None:
+def register_architecture(name: str, config_reader: Callable[[Mapping[str, Any]], Any],
+                          sizes_from_tensors: bool = False) -> None:
     """`config_reader(dict)` returns an object with `.plan() -> ModelPlan` and
-    `.to_json_dict() -> dict` (the config.json it would be read from)."""
+    `.to_json_dict() -> dict` (the config.json it would be read from).  With `sizes_from_tensors` the
+    reader is called as `config_reader(dict, shapes)`, `shapes` the checkpoint's {tensor name: shape} when the
+    config comes from a model folder and None when it comes from a dict alone."""
     _ARCHITECTURES[name] = config_reader
+    if sizes_from_tensors:
+        _READS_SHAPES.add(name)
 
 
 def known_architectures():
     return tuple(sorted(_ARCHITECTURES))
 
 
-def read_config_dict(cfg: Mapping[str, Any]):
+def read_config_dict(cfg: Mapping[str, Any], shapes=None):
     archs = cfg.get("architectures")
     if not archs and isinstance(cfg.get("architecture"), str):
         archs = [cfg["architecture"]]  # some configurations name their one architecture in the singular
@@ -37,7 +44,14 @@ def read_config_dict(cfg: Mapping[str, Any]):
     if name not in _ARCHITECTURES:
         raise ConfigError(
             f"unknown architecture '{name}'; known: {', '.join(known_architectures()) or '(none)'}")
+    if name in _READS_SHAPES:
+        return _ARCHITECTURES[name](cfg, shapes)
     return _ARCHITECTURES[name](cfg)
+
+
+def _architecture_of(cfg: Mapping[str, Any]):
+    archs = cfg.get("architectures") or ([cfg["architecture"]] if isinstance(cfg.get("architecture"), str) else None)
+    return archs[0] if isinstance(archs, (list, tuple)) and archs else None
 
 
 def read_config(model_dir: str):
@@ -50,7 +64,14 @@ def read_config(model_dir: str):
         raise ConfigError(f"{path}: no such file") from err
     except json.JSONDecodeError as err:
         raise ConfigError(f"{path}: not JSON ({err})") from err
-    return read_config_dict(cfg)
+    shapes = None
+    if _architecture_of(cfg) in _READS_SHAPES:
+        from ..weights.loader import WeightsError, stored_shapes
+        try:
+            shapes = stored_shapes(model_dir)
+        except WeightsError:
+            shapes = None  # a folder without weights: the config must name those sizes itself
+    return read_config_dict(cfg, shapes)
 
 
 def plan_of(model_dir_or_dict) -> ModelPlan:

@@ -115,8 +115,34 @@ int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stride, int num
                         float* conv_tail, int64_t tail_slot_stride, int taps, int G, int H, int D, int V,
                         const float* a_log, const float* dt_bias, float unit_eps, float* state,
                         int64_t state_slot_stride, const void* norm_w, int w_is_f32, float norm_eps, float* work,
-                        void* out, hipStream_t stream);
-int64_t pae_delta_rule_work_floats(int num_tokens, int G, int H, int D, int V);
+                        void* out, const void* gate_in, int64_t gate_stride, int gate_sigmoid, const void* b_in,
+                        int64_t b_stride, const void* a_in, int64_t a_stride, int channel_decay, hipStream_t stream);
+int64_t pae_delta_rule_work_floats(int num_tokens, int G, int H, int D, int V, int channel_decay);
+// a matrix memory with exponential gates over a step's projected rows: see matrix_memory.hip
+int pae_matrix_memory_step(int dtype, const void* proj, int64_t row_stride, const void* gate_in, int64_t gate_stride,
+                           const float* gate_logits, int num_tokens, int num_seqs, const int* seq_runs, const int* slots,
+                           int H, int D, int V, float gate_cap, float* state, int64_t state_slot_stride, float* maximum,
+                           int64_t max_slot_stride, const void* norm_w, int w_is_f32, float norm_eps, float floor_eps,
+                           float* work, void* out, hipStream_t stream);
+int64_t pae_matrix_memory_work_floats(int num_tokens, int H, int D, int V);
+// the embedding with a hashed table of token pairs added: see hashed_embedding.hip
+int pae_embedding_pairs(int dtype, float* out, const void* table, const void* pair_table, const int* ids,
+                        const int* positions, const int* tok_seq, const int* slots, int* last_token, int num_tokens,
+                        int hidden, int vocab, float scale, int buckets, int mul_prev, int mul_cur, hipStream_t stream);
+// residual += terms; two norms of the new residual: see parallel_norm.hip
+int pae_sum_norm2(int dtype, float* residual, int num_terms, const void* const* term_ptr, const int* term_is_f32,
+                  const int* term_parts, const int64_t* term_part_stride, const float* term_scale, const void* w1,
+                  int w1_is_f32, const void* w2, int w2_is_f32, float eps, const int* rows, void* out1, void* out2,
+                  int num_rows, int hidden, int write_residual, hipStream_t stream);
+// float32 sums of a few output features from rows of either type: see moe.hip
+int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* bias,
+                    int b_is_f32, int M, int N, int K, hipStream_t stream);
+int pae_moe_route(const float* logits, int num_tokens, int experts, int groups, int keep, int top, float scale,
+                  int* chosen, float* weights, hipStream_t stream);
+int pae_moe_gate_up(int dtype, void* act, const void* x, int64_t ldx, const void* gate_w, const void* up_w,
+                    const int* chosen, int num_tokens, int top, int hidden, int inter, int act_kind, hipStream_t stream);
+int pae_moe_down(int dtype, float* out, const void* act, const void* down_w, const int* chosen, const float* weights,
+                 int num_tokens, int top, int hidden, int inter, hipStream_t stream);
 int pae_attn_decode_split();
 int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                          const void* v_cache, const int* dec_work, int num_dec, const int* block_tables,

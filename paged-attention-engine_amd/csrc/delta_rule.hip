@@ -17,6 +17,13 @@
 //                      first token to its last; the lanes of a group share out the D rows.
 //   delta_gated_norm   o / sqrt(mean_V(o^2) + eps) * w * silu(gate), rounded to the activation type.
 //
+// For designs that have them, each switched by a parameter: a decay per head and key channel instead of one
+// per head (`channel_decay`: the decay's input and dt_bias are then H x D wide and row d of a head's S is
+// multiplied by its own number); beta, the decay's input and the gate read from rows of their own instead of
+// the projected rows' tail (a design whose decay and gate pass through a narrow product first); sigmoid
+// instead of SiLU on the gate.  The recurrence kernels also run a matrix memory that only adds
+// (`delta` off: u = beta v, nothing is read back before the write; see matrix_memory.hip).
+//
 // Everything but the projected rows is float32: the convolution's sums, the unit vectors, beta,
 // the decay and its logarithm, the state, the read-out and the norm.  The order in which a
 // column's sums are formed depends on D alone, so a token's result does not depend on how a
@@ -35,7 +42,8 @@ __global__ __launch_bounds__(128) void delta_prepare_kernel(
     const T* __restrict__ proj, int64_t row_stride, const int* __restrict__ tok_seq, const int* __restrict__ positions,
     const int4* __restrict__ seq_runs, const int* __restrict__ slots, const float* __restrict__ conv_w,
     const float* __restrict__ conv_tail, int64_t tail_slot_stride, int taps, int G, int H, int D, int V,
-    const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps, float* __restrict__ q_out,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps, const T* __restrict__ b_in,
+    int64_t b_stride, const T* __restrict__ a_in, int64_t a_stride, int channel_decay, float* __restrict__ q_out,
     float* __restrict__ k_out, float* __restrict__ v_out, float* __restrict__ beta_out, float* __restrict__ decay_out) {
   __shared__ float scratch[2];
   const int t = blockIdx.x, seg = blockIdx.y;
@@ -82,11 +90,15 @@ __global__ __launch_bounds__(128) void delta_prepare_kernel(
     dst[i] = is_v ? mine[n] : (seg < G ? mine[n] * inv * q_scale : mine[n] * inv);
   }
   if (seg == 0) {
-    const T* row = proj + (int64_t)t * row_stride;
-    for (int h = threadIdx.x; h < H; h += 128) {
-      const float b = to_f32(row[C + H * V + h]), a = to_f32(row[C + H * V + H + h]);
-      beta_out[(int64_t)t * H + h] = 1.0f / (1.0f + expf(-b));
-      decay_out[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
+    const T* b_row = b_in + (int64_t)t * b_stride;
+    const T* a_row = a_in + (int64_t)t * a_stride;
+    for (int h = threadIdx.x; h < H; h += 128) beta_out[(int64_t)t * H + h] = 1.0f / (1.0f + expf(-to_f32(b_row[h])));
+    if (channel_decay) {  // one decay per head and key channel, [H][D]
+      for (int c = threadIdx.x; c < H * D; c += 128)
+        decay_out[(int64_t)t * H * D + c] = expf(-expf(a_log[c / D]) * softplus_f(to_f32(a_row[c]) + dt_bias[c]));
+    } else {
+      for (int h = threadIdx.x; h < H; h += 128)
+        decay_out[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(to_f32(a_row[h]) + dt_bias[h]));
     }
   }
 }
@@ -114,7 +126,8 @@ template <int R>
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ decay, const int4* __restrict__ seq_runs, const int* __restrict__ slots,
-    float* __restrict__ state, int64_t state_slot_stride, int G, int H, int D, int V, int L, float* __restrict__ out) {
+    float* __restrict__ state, int64_t state_slot_stride, int G, int H, int D, int V, int L, int channel_decay, int delta,
+    float* __restrict__ out) {
   const int s = blockIdx.z, h = blockIdx.y;
   const int col = blockIdx.x * (256 / L) + threadIdx.x / L;
   const int sub = threadIdx.x % L;
@@ -139,15 +152,17 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
       kr[r] = d < D ? kt[d] : 0.f;
       qr[r] = d < D ? qt[d] : 0.f;
     }
-    const float dec = decay[t * H + h], b = beta[t * H + h], vt = v[(t * H + h) * V + col];
+    const float dec = channel_decay ? 0.f : decay[t * H + h], b = beta[t * H + h], vt = v[(t * H + h) * V + col];
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      S[r] = dec * S[r];
+      const int d = sub * R + r;
+      const float dr = channel_decay ? (d < D ? decay[(t * H + h) * D + d] : 0.f) : dec;
+      S[r] = dr * S[r];
       dot = fmaf(S[r], kr[r], dot);
     }
     for (int off = L / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, L);
-    const float u = b * (vt - dot);
+    const float u = delta ? b * (vt - dot) : b * vt;
     float o = 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -181,7 +196,7 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int R, int L, int CH>
+template <int R, int L, int CH, bool CHANNEL, bool DELTA>
 __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ decay, const int4* __restrict__ seq_runs, const int* __restrict__ slots,
@@ -193,8 +208,9 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
   static_assert(R % 4 == 0 && CH * DP % (4 * NT) == 0 && CH * 16 % NT == 0 && 2 * CH <= NT, "chunk shape");
   __shared__ __attribute__((aligned(16))) float s_k[CH * DP];
   __shared__ __attribute__((aligned(16))) float s_q[CH * DP];
+  __shared__ __attribute__((aligned(16))) float s_dec[CHANNEL ? CH * DP : 4];  // a decay per key channel
   __shared__ float s_v[CH * 16];
-  __shared__ float s_bd[2 * CH];     // beta, then decay
+  __shared__ float s_bd[2 * CH];     // beta, then decay (one per head)
   const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * 16;
   const int tid = threadIdx.x;
   const int col = col0 + tid / L, sub = tid % L;
@@ -209,7 +225,7 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
     S[r] = (live && d < D) ? column[d] : 0.f;
   }
   const bool vec = D % 4 == 0;
-  float pk[KQ], pq[KQ], pv[VN], pbd;
+  float pk[KQ], pq[KQ], pd[CHANNEL ? KQ : 1], pv[VN], pbd;
   // a thread's share of the chunk that starts at token `first` of the run, from memory into registers
   auto fetch = [&](int first) {
     if (vec) {
@@ -224,6 +240,12 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
         }
         pk[4 * p] = a.x; pk[4 * p + 1] = a.y; pk[4 * p + 2] = a.z; pk[4 * p + 3] = a.w;
         pq[4 * p] = b.x; pq[4 * p + 1] = b.y; pq[4 * p + 2] = b.z; pq[4 * p + 3] = b.w;
+        if (CHANNEL) {
+          float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (first + i < run.y && d < D)
+            c = *reinterpret_cast<const float4*>(decay + ((int64_t)(run.x + first + i) * H + h) * D + d);
+          pd[4 * p] = c.x; pd[4 * p + 1] = c.y; pd[4 * p + 2] = c.z; pd[4 * p + 3] = c.w;
+        }
       }
     } else {
 #pragma unroll
@@ -233,6 +255,7 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
         const int64_t at = ((int64_t)(run.x + first + i) * G + g) * D + d;
         pk[p] = there ? k[at] : 0.f;
         pq[p] = there ? q[at] : 0.f;
+        if (CHANNEL) pd[p] = there ? decay[((int64_t)(run.x + first + i) * H + h) * D + d] : 0.f;
       }
     }
 #pragma unroll
@@ -241,7 +264,7 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
       pv[p] = (first + i < run.y && c < V) ? v[((int64_t)(run.x + first + i) * H + h) * V + c] : 0.f;
     }
     pbd = 0.f;
-    if (tid < 2 * CH && first + tid % CH < run.y)
+    if (tid < (CHANNEL ? CH : 2 * CH) && first + tid % CH < run.y)
       pbd = (tid < CH ? beta : decay)[(int64_t)(run.x + first + tid % CH) * H + h];
   };
   auto stage = [&]() {
@@ -251,12 +274,14 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
         const int e = (tid + NT * p) * 4;
         *reinterpret_cast<float4*>(s_k + e) = make_float4(pk[4 * p], pk[4 * p + 1], pk[4 * p + 2], pk[4 * p + 3]);
         *reinterpret_cast<float4*>(s_q + e) = make_float4(pq[4 * p], pq[4 * p + 1], pq[4 * p + 2], pq[4 * p + 3]);
+        if (CHANNEL) *reinterpret_cast<float4*>(s_dec + e) = make_float4(pd[4 * p], pd[4 * p + 1], pd[4 * p + 2], pd[4 * p + 3]);
       }
     } else {
 #pragma unroll
       for (int p = 0; p < KQ; ++p) {
         s_k[tid + NT * p] = pk[p];
         s_q[tid + NT * p] = pq[p];
+        if (CHANNEL) s_dec[tid + NT * p] = pd[p];
       }
     }
 #pragma unroll
@@ -281,13 +306,22 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
         const float4 k4 = *reinterpret_cast<const float4*>(kt + r4 * (4 * L) + sub * 4);
         kr[4 * r4] = k4.x; kr[4 * r4 + 1] = k4.y; kr[4 * r4 + 2] = k4.z; kr[4 * r4 + 3] = k4.w;
       }
+      if (CHANNEL) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        S[r] = dec * S[r];
-        dot = fmaf(S[r], kr[r], dot);
+        for (int r4 = 0; r4 < R / 4; ++r4) {
+          const float4 d4 = *reinterpret_cast<const float4*>(s_dec + i * DP + r4 * (4 * L) + sub * 4);
+          S[4 * r4] *= d4.x; S[4 * r4 + 1] *= d4.y; S[4 * r4 + 2] *= d4.z; S[4 * r4 + 3] *= d4.w;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) S[r] = dec * S[r];
       }
-      dot = group_sum<L>(dot);
-      const float u = b * (vt - dot);
+      if (DELTA) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) dot = fmaf(S[r], kr[r], dot);
+        dot = group_sum<L>(dot);
+      }
+      const float u = DELTA ? b * (vt - dot) : b * vt;
       float o = 0.f;
 #pragma unroll
       for (int r4 = 0; r4 < R / 4; ++r4) {
@@ -311,8 +345,8 @@ __global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
 }
 
 template <typename T>
-__global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const T* __restrict__ proj,
-                                                                    int64_t row_stride, int gate_offset,
+__global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const T* __restrict__ gates,
+                                                                    int64_t gate_stride, int gate_sigmoid,
                                                                     const void* __restrict__ weight, int w_is_f32, float eps,
                                                                     int H, int V, T* __restrict__ out) {
   const int64_t t = blockIdx.x;
@@ -322,21 +356,36 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float*
   for (int i = lane; i < V; i += PAE_WAVE) ss = fmaf(x[i], x[i], ss);
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)V + eps);
-  const T* gate = proj + t * row_stride + gate_offset + h * V;
-  for (int i = lane; i < V; i += PAE_WAVE)
-    out[(t * H + h) * V + i] = from_f32<T>(x[i] * inv * load_param(weight, w_is_f32, i) * silu_f(to_f32(gate[i])));
+  const T* gate = gates + t * gate_stride + h * V;
+  for (int i = lane; i < V; i += PAE_WAVE) {
+    const float z = to_f32(gate[i]);
+    const float gz = gate_sigmoid ? 1.0f / (1.0f + expf(-z)) : silu_f(z);
+    out[(t * H + h) * V + i] = from_f32<T>(x[i] * inv * load_param(weight, w_is_f32, i) * gz);
+  }
 }
 
 static int lanes_per_column(int D, int R);
+void pae_launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
+                           const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,
+                           int D, int V, int num_seqs, int channel_decay, int delta, float* o, hipStream_t stream);
 
-static void launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
-                              const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,
-                              int D, int V, int num_seqs, float* o, hipStream_t stream) {
+// The recurrence over a step's rows for every (sequence, head, column of S).  `channel_decay`: `decay` is
+// [T][H][D] instead of [T][H]; `delta` off: u = beta v (a memory that only adds).
+void pae_launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
+                           const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,
+                           int D, int V, int num_seqs, int channel_decay, int delta, float* o, hipStream_t stream) {
   dim3 group_grid((V + 15) / 16, H, num_seqs);
   // (rows a lane, lanes a column, tokens a chunk)
-#define GROUP(R, L, CH)                                                                                          \
-  delta_recurrence_group_kernel<R, L, CH><<<group_grid, 16 * L, 0, stream>>>(q, k, v, beta, decay, runs, slots, state, \
-                                                                             state_slot_stride, G, H, D, V, o)
+#define GROUP_AS(R, L, CH, CHANNEL, DELTA)                                                                        \
+  delta_recurrence_group_kernel<R, L, CH, CHANNEL, DELTA><<<group_grid, 16 * L, 0, stream>>>(                     \
+      q, k, v, beta, decay, runs, slots, state, state_slot_stride, G, H, D, V, o)
+#define GROUP(R, L, CH)                                       \
+  do {                                                        \
+    if (channel_decay && delta) GROUP_AS(R, L, CH, true, true);      \
+    else if (channel_decay) GROUP_AS(R, L, CH, true, false);  \
+    else if (delta) GROUP_AS(R, L, CH, false, true);          \
+    else GROUP_AS(R, L, CH, false, false);                    \
+  } while (0)
   if (D <= 16) GROUP(4, 4, 32);
   else if (D <= 32) GROUP(8, 4, 32);
   else if (D <= 64) GROUP(8, 8, 16);
@@ -346,9 +395,10 @@ static void launch_recurrence(const float* q, const float* k, const float* v, co
     const int L = lanes_per_column(D, 16);
     dim3 rec_grid((V + 256 / L - 1) / (256 / L), H, num_seqs);
     delta_recurrence_kernel<16><<<rec_grid, 256, 0, stream>>>(q, k, v, beta, decay, runs, slots, state,
-                                                              state_slot_stride, G, H, D, V, L, o);
+                                                              state_slot_stride, G, H, D, V, L, channel_decay, delta, o);
   }
 #undef GROUP
+#undef GROUP_AS
 }
 
 static int lanes_per_column(int D, int R) {
@@ -357,41 +407,49 @@ static int lanes_per_column(int D, int R) {
   return L;
 }
 
+static int64_t work_part(int64_t floats) { return (floats + 3) / 4 * 4; }
+
 extern "C" int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stride, int num_tokens, int num_seqs,
                                    const int* tok_seq, const int* positions, const int* seq_runs, const int* slots,
                                    const float* conv_w, float* conv_tail, int64_t tail_slot_stride, int taps, int G,
                                    int H, int D, int V, const float* a_log, const float* dt_bias, float unit_eps,
                                    float* state, int64_t state_slot_stride, const void* norm_w, int w_is_f32,
-                                   float norm_eps, float* work, void* out, hipStream_t stream) {
+                                   float norm_eps, float* work, void* out, const void* gate_in, int64_t gate_stride,
+                                   int gate_sigmoid, const void* b_in, int64_t b_stride, const void* a_in, int64_t a_stride,
+                                   int channel_decay, hipStream_t stream) {
   PAE_REQUIRE(G > 0 && H > 0 && H % G == 0 && D > 0 && V > 0, "delta rule: bad head sizes G=%d H=%d D=%d V=%d", G, H, D, V);
   PAE_REQUIRE(taps >= 1 && taps <= 64, "delta rule: %d convolution taps", taps);
   PAE_REQUIRE(D <= 1024, "delta rule: key width %d exceeds 1024", D);
   PAE_REQUIRE(H <= 65535 && num_seqs <= 65535, "delta rule: %d heads, %d sequences exceed the grid", H, num_seqs);
   const int64_t C = 2 * (int64_t)G * D + (int64_t)H * V;
   PAE_REQUIRE(V <= 1024 && 2 * G + H <= 65535, "delta rule: value width %d or %d heads exceed the kernels' limits", V, 2 * G + H);
-  PAE_REQUIRE(row_stride >= C + (int64_t)H * V + 2 * H, "delta rule: row stride %lld too small", (long long)row_stride);
+  PAE_REQUIRE(row_stride >= C, "delta rule: row stride %lld too small", (long long)row_stride);
+  PAE_REQUIRE(gate_in && b_in && a_in, "delta rule: the gate's, beta's and the decay's rows are needed");
   PAE_REQUIRE(dtype == PAE_F32 || dtype == PAE_BF16, "delta rule: unknown dtype code %d", dtype);
   if (num_tokens <= 0 || num_seqs <= 0) return 0;
-  // work: q [T][G][D], k [T][G][D], v [T][H][V], beta [T][H], decay [T][H], o [T][H][V]
+  // work: q [T][G][D], k [T][G][D], v [T][H][V], beta [T][H], decay [T][H] or [T][H][D], o [T][H][V]
+  // (every part starts on a 16-byte boundary: the recurrence reads k, q and channel decays four at a time)
   float* q = work;
-  float* k = q + (int64_t)num_tokens * G * D;
-  float* v = k + (int64_t)num_tokens * G * D;
-  float* beta = v + (int64_t)num_tokens * H * V;
-  float* decay = beta + (int64_t)num_tokens * H;
-  float* o = decay + (int64_t)num_tokens * H;
+  float* k = q + work_part((int64_t)num_tokens * G * D);
+  float* v = k + work_part((int64_t)num_tokens * G * D);
+  float* beta = v + work_part((int64_t)num_tokens * H * V);
+  float* decay = beta + work_part((int64_t)num_tokens * H);
+  float* o = decay + work_part((int64_t)num_tokens * H * (channel_decay ? D : 1));
   const int4* runs = (const int4*)seq_runs;
   dim3 tail_grid((unsigned)((C + 255) / 256), num_seqs);
   dim3 norm_grid(num_tokens, H);
 #define DELTA_LAUNCH(T)                                                                                                 \
   delta_prepare_kernel<T><<<dim3(num_tokens, 2 * G + H), 128, 0, stream>>>(                                             \
       (const T*)proj, row_stride, tok_seq, positions, runs, slots, conv_w, conv_tail, tail_slot_stride, taps, G, H, D,  \
-      V, a_log, dt_bias, unit_eps, q, k, v, beta, decay);                                                               \
+      V, a_log, dt_bias, unit_eps, (const T*)b_in, b_stride, (const T*)a_in, a_stride, channel_decay, q, k, v, beta,    \
+      decay);                                                                                                           \
   if (taps > 1)                                                                                                         \
     delta_conv_tail_kernel<T><<<tail_grid, 256, 0, stream>>>((const T*)proj, row_stride, runs, slots, conv_tail,        \
                                                              tail_slot_stride, taps, (int)C);                           \
-  launch_recurrence(q, k, v, beta, decay, runs, slots, state, state_slot_stride, G, H, D, V, num_seqs, o, stream);      \
-  delta_gated_norm_kernel<T><<<norm_grid, PAE_WAVE, 0, stream>>>(o, (const T*)proj, row_stride, (int)C, norm_w,         \
-                                                                 w_is_f32, norm_eps, H, V, (T*)out)
+  pae_launch_recurrence(q, k, v, beta, decay, runs, slots, state, state_slot_stride, G, H, D, V, num_seqs,              \
+                        channel_decay, 1, o, stream);                                                                   \
+  delta_gated_norm_kernel<T><<<norm_grid, PAE_WAVE, 0, stream>>>(o, (const T*)gate_in, gate_stride, gate_sigmoid,       \
+                                                                 norm_w, w_is_f32, norm_eps, H, V, (T*)out)
   if (dtype == PAE_F32) {
     DELTA_LAUNCH(float);
   } else {
@@ -402,6 +460,7 @@ extern "C" int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stri
 }
 
 // floats of `work` that pae_delta_rule_step needs for a step of `num_tokens` rows
-extern "C" int64_t pae_delta_rule_work_floats(int num_tokens, int G, int H, int D, int V) {
-  return (int64_t)num_tokens * (2 * (int64_t)G * D + 2 * (int64_t)H * V + 2 * H);
+extern "C" int64_t pae_delta_rule_work_floats(int num_tokens, int G, int H, int D, int V, int channel_decay) {
+  const int64_t T = num_tokens;
+  return 2 * work_part(T * G * D) + 2 * work_part(T * H * V) + work_part(T * H) + work_part(T * H * (channel_decay ? D : 1));
 }

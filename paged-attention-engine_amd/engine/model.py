@@ -16,7 +16,7 @@ from typing import Dict, List, Mapping, Optional, Tuple
 import torch
 
 from .. import models as _models  # noqa: F401  (registers the architectures)
-from ..cache.manager import CacheManager, bytes_of_one_page_everywhere
+from ..cache.manager import CacheManager, StateSpec, bytes_of_one_page_everywhere
 from ..config.model_config import ModelPlan
 from ..config.registry import read_config, read_config_dict
 from ..kernels import lib as K
@@ -54,6 +54,8 @@ def expected_tensors(plan: ModelPlan) -> Dict[str, Tuple[int, ...]]:
     out.update(build_part(NORMS, "norm", plan.final_norm, torch.float32, "meta").tensors(plan.final_norm_prefix))
     if plan.head_name is not None:
         out[plan.head_name] = (plan.vocab_size, plan.hidden_size)
+    if plan.pair_embedding is not None:
+        out[plan.pair_embedding.name] = (plan.pair_embedding.buckets + 1, plan.hidden_size)
     return out
 
 
@@ -82,6 +84,9 @@ class Model:
         plan = self.plan
         embedding = weights[plan.embedding_name]
         self.embedding = embedding.to(device=self.device, dtype=self.dtype).contiguous()
+        self.pair_table = None
+        if plan.pair_embedding is not None:
+            self.pair_table = weights[plan.pair_embedding.name].to(device=self.device, dtype=self.dtype).contiguous()
         for block in self.blocks:
             block.bind(weights)
         self.final_norm.bind(plan.final_norm_prefix, weights)
@@ -114,7 +119,10 @@ class Model:
         """key -> the first part that asks for index lists under that key (see `Part.step_lists`)."""
         out: Dict[object, object] = {}
         for block in self.blocks:
-            for part in getattr(block, "parts", lambda: [])():
+            listed = list(getattr(block, "parts", lambda: [])())
+            for part in listed:  # a part made of parts (mixers side by side) names them
+                listed.extend(getattr(part, "inner_parts", lambda: [])())
+            for part in listed:
                 key = part.step_lists_key(block_size) if hasattr(part, "step_lists_key") else None
                 if key is not None and key not in out:
                     out[key] = part
@@ -131,7 +139,15 @@ class Model:
             # a mixer that says so keeps state of its own at a stop that borrows its pages (the inputs of
             # convolutions on its queries, say)
             states.append(mixer.state_spec() if not borrowed or getattr(mixer, "state_when_borrowing", False) else None)
+        if self.plan.pair_embedding is not None:
+            # what the embedding keeps per request (the token before the next one) lives behind the last stop
+            paged.append(None)
+            states.append(StateSpec((), torch.int32, "last_token"))
         return paged, states
+
+    @property
+    def embedding_state_entry(self) -> int:
+        return len(self.plan.schedule)
 
     def page_bytes(self, block_size: int) -> int:
         """Bytes of one page in every cache group of this model (all stops)."""
@@ -185,7 +201,7 @@ class Model:
         # the norm that reads the stream first at every stop (and the final norm after the last)
         first_norms = [getattr(self.blocks[entry.layer], "mixer_norm", None) for entry in plan.schedule] + [self.final_norm]
         entry_fold = getattr(self.blocks[plan.schedule[0].layer], "entry_fold", None) if plan.schedule and T else None
-        fold = entry_fold(T) if entry_fold is not None else None
+        fold = entry_fold(T) if entry_fold is not None and plan.pair_embedding is None else None
         if fold is not None:
             # the first block's norm lets the embedding prepare its rows (see parts.OwedRows)
             norm, weight, eps = fold
@@ -193,6 +209,13 @@ class Model:
             stats = torch.empty((T, K.stat_tiles(H)), dtype=torch.float32, device=self.device)
             K.embedding_rows(residual, self.embedding, token_ids, plan.embedding_scale, rows, weight, stats)
             stream.owed, stream.owed_to = OwedRows(rows, stats, eps), norm
+        elif plan.pair_embedding is not None:
+            pairs = plan.pair_embedding
+            K.embedding_pairs(residual, self.embedding, self.pair_table, token_ids, ctx.positions, ctx.tok_seq, ctx.slots,
+                              ctx.cache.state_of(self.embedding_state_entry), plan.embedding_scale, pairs.buckets,
+                              pairs.mul_prev, pairs.mul_cur)
+            if copies > 1:
+                K.hyper_spread(stream.residual, residual, copies)
         else:
             K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
             if copies > 1:

@@ -89,7 +89,15 @@ def _declare(lib) -> None:
         "pae_rows_from_residual": [I, P, P, L, P],
         "pae_norm_scale_add": [I, P, P, I, L, P, I, F, F, P, I, I, P],
         "pae_activation": [I, P, L, I, P],
-        "pae_delta_rule_step": [I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, P, P, F, P, L, P, I, F, P, P, P],
+        "pae_delta_rule_step": [I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, P, P, F, P, L, P, I, F, P, P,
+                                P, L, I, P, L, P, L, I, P],
+        "pae_matrix_memory_step": [I, P, L, P, L, P, I, I, P, P, I, I, I, F, P, L, P, L, P, I, F, F, P, P, P],
+        "pae_embedding_pairs": [I, P, P, P, P, P, P, P, P, I, I, I, F, I, I, I, P],
+        "pae_sum_norm2": [I, P, I, P, P, P, P, P, P, I, P, I, F, P, P, P, I, I, I, P],
+        "pae_project_f32": [I, P, L, P, L, P, P, I, I, I, I, P],
+        "pae_moe_route": [P, I, I, I, I, I, F, P, P, P],
+        "pae_moe_gate_up": [I, P, P, L, P, P, P, I, I, I, I, I, P],
+        "pae_moe_down": [I, P, P, P, P, P, I, I, I, I, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
         "pae_sample_chunks": [I],
         "pae_sample_static": [P, P, L, P, P, I, I, P],
@@ -120,8 +128,10 @@ def _declare(lib) -> None:
         fn.restype = c_int
     lib.pae_skinny_ticket_floats.argtypes = [I, I, I]
     lib.pae_skinny_ticket_floats.restype = c_int64
-    lib.pae_delta_rule_work_floats.argtypes = [I, I, I, I, I]
+    lib.pae_delta_rule_work_floats.argtypes = [I, I, I, I, I, I]
     lib.pae_delta_rule_work_floats.restype = c_int64
+    lib.pae_matrix_memory_work_floats.argtypes = [I, I, I, I]
+    lib.pae_matrix_memory_work_floats.restype = c_int64
 
 
 def _check(code: int) -> None:
@@ -547,7 +557,7 @@ def scaled_rows(rows: torch.Tensor, stats: torch.Tensor, eps: float) -> torch.Te
 def skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
     """The weight-streaming product takes bfloat16, at most 64 rows and rows of 16-byte multiples."""
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_ROWS
-            and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.stride(1) == 1)
+            and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.stride(1) == 1 and a.data_ptr() % 16 == 0)
 
 
 def skinny_splits(N: int, K: int, M: int = 1) -> int:
@@ -1313,17 +1323,32 @@ def activation(x: torch.Tensor, kind: str) -> None:
 def delta_rule_step(proj: torch.Tensor, out: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
                     seq_runs: torch.Tensor, slots: torch.Tensor, conv_w: torch.Tensor, conv_tail: torch.Tensor,
                     state: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, norm_w: torch.Tensor,
-                    G: int, H: int, D: int, V: int, taps: int, unit_eps: float, norm_eps: float) -> None:
-    """The gated delta rule over a step's rows.  `proj` [T, 2GD + 2HV + 2H] holds per token
-    [q | k | v | gate | b | a]; `seq_runs` int32 [S, 4] = (first row, rows, tokens before, 0) per
-    sequence; `slots` int32 [S]; `conv_w` float32 [2GD + HV, taps]; `conv_tail` float32
-    [slots, taps - 1, 2GD + HV] and `state` float32 [slots, H, V, D] are the requests' state, read
-    and moved on; `out` [T, H * V] receives the normed, gated read-out in proj's type."""
+                    G: int, H: int, D: int, V: int, taps: int, unit_eps: float, norm_eps: float,
+                    gate: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None,
+                    decay_in: Optional[torch.Tensor] = None, channel_decay: bool = False,
+                    gate_activation: str = "silu") -> None:
+    """The gated delta rule over a step's rows.  `proj` [T, >= 2GD + HV] holds per token [q | k | v | ...];
+    the gate's rows [T, HV], beta's [T, H] and the decay's input [T, H] come as views of rows in proj's type
+    (`gate`, `beta`, `decay_in`), or, when none is given, from proj's tail [gate | b | a].  `seq_runs` int32
+    [S, 4] = (first row, rows, tokens before, 0) per sequence; `slots` int32 [S]; `conv_w` float32
+    [2GD + HV, taps]; `conv_tail` float32 [slots, taps - 1, 2GD + HV] and `state` float32 [slots, H, V, D] are
+    the requests' state, read and moved on; `out` [T, H * V] receives the normed, gated read-out in proj's type.
+    `channel_decay`: one decay per head and key channel (`decay_in` [T, H * D], `dt_bias` [H * D]) instead of
+    one per head; `gate_activation`: "silu" or "sigmoid"."""
     _not_while_recording("delta_rule_step")
-    _gpu(proj, out, tok_seq, positions, seq_runs, slots, conv_w, conv_tail, state, a_log, dt_bias, norm_w)
+    _gpu(proj, out, tok_seq, positions, seq_runs, slots, conv_w, conv_tail, state, a_log, dt_bias, norm_w, gate, beta,
+         decay_in)
     T, S = proj.shape[0], seq_runs.shape[0]
     C = 2 * G * D + H * V
-    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] == C + H * V + 2 * H
+    assert gate_activation in ("silu", "sigmoid")
+    assert proj.dim() == 2 and proj.stride(1) == 1
+    if gate is None and beta is None and decay_in is None:
+        assert proj.shape[1] == C + H * V + 2 * H and not channel_decay
+        gate, beta, decay_in = proj[:, C:C + H * V], proj[:, C + H * V:C + H * V + H], proj[:, C + H * V + H:]
+    assert proj.shape[1] >= C
+    for view, width in ((gate, H * V), (beta, H), (decay_in, H * D if channel_decay else H)):
+        assert view is not None and view.dim() == 2 and view.shape == (T, width) and view.dtype == proj.dtype
+        assert view.stride(1) == 1 or width == 1
     assert out.shape == (T, H * V) and out.is_contiguous() and out.dtype == proj.dtype
     for t, n in ((tok_seq, T), (positions, T), (slots, S)):
         assert t.dtype == torch.int32 and t.numel() >= n and t.is_contiguous()
@@ -1334,17 +1359,171 @@ def delta_rule_step(proj: torch.Tensor, out: torch.Tensor, tok_seq: torch.Tensor
     assert conv_tail.stride(2) == 1 and (taps == 1 or conv_tail.stride(1) == C)
     assert state.dtype == torch.float32 and tuple(state.shape[1:]) == (H, V, D) and state[0].is_contiguous()
     assert state.shape[0] == conv_tail.shape[0]
-    for t in (a_log, dt_bias):
-        assert t.dtype == torch.float32 and t.numel() == H and t.is_contiguous()
+    assert a_log.dtype == torch.float32 and a_log.numel() == H and a_log.is_contiguous()
+    assert dt_bias.dtype == torch.float32 and dt_bias.numel() == (H * D if channel_decay else H) and dt_bias.is_contiguous()
     assert norm_w.numel() == V
     wp, wf = _param(norm_w)
     lib = library()
-    work = torch.empty(lib.pae_delta_rule_work_floats(T, G, H, D, V), dtype=torch.float32, device=proj.device)
+    work = torch.empty(lib.pae_delta_rule_work_floats(T, G, H, D, V, 1 if channel_decay else 0), dtype=torch.float32,
+                       device=proj.device)
     _check(lib.pae_delta_rule_step(
         code_of(proj.dtype), proj.data_ptr(), proj.stride(0), T, S, tok_seq.data_ptr(), positions.data_ptr(),
         seq_runs.data_ptr(), slots.data_ptr(), conv_w.data_ptr(), conv_tail.data_ptr(), conv_tail.stride(0), taps, G, H,
         D, V, a_log.data_ptr(), dt_bias.data_ptr(), float(unit_eps), state.data_ptr(), state.stride(0), wp, wf,
-        float(norm_eps), work.data_ptr(), out.data_ptr(), _stream()))
+        float(norm_eps), work.data_ptr(), out.data_ptr(), gate.data_ptr(), gate.stride(0),
+        1 if gate_activation == "sigmoid" else 0, beta.data_ptr(), beta.stride(0), decay_in.data_ptr(), decay_in.stride(0),
+        1 if channel_decay else 0, _stream()))
+
+
+def matrix_memory_step(proj: torch.Tensor, gate: torch.Tensor, gate_logits: torch.Tensor, out: torch.Tensor,
+                       seq_runs: torch.Tensor, slots: torch.Tensor, state: torch.Tensor, maximum: torch.Tensor,
+                       norm_w: torch.Tensor, H: int, D: int, V: int, gate_cap: float, norm_eps: float,
+                       floor_eps: float) -> None:
+    """A matrix memory with exponential gates over a step's rows.  `proj` [T, >= 2HD + HV] holds per token
+    [q | k | v]; `gate` [T, HV] (a view of rows in proj's type) is the output gate's input; `gate_logits` float32
+    [T, 2H] the input and forget gates' sums with their biases.  `state` float32 [slots, H, V + 1, D] (the
+    memory, and as its last column the sum of gated keys) and `maximum` float32 [slots, H] are the requests'
+    state, read and moved on; `out` [T, H * V] receives o / (max(|n . q|, exp(-m)) + floor_eps), normed over V,
+    times `norm_w` [H * V] and sigmoid(gate), in proj's type."""
+    _not_while_recording("matrix_memory_step")
+    _gpu(proj, gate, gate_logits, out, seq_runs, slots, state, maximum, norm_w)
+    T, S = proj.shape[0], seq_runs.shape[0]
+    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= 2 * H * D + H * V
+    assert gate.shape == (T, H * V) and gate.stride(1) == 1 and gate.dtype == proj.dtype
+    assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, 2 * H) and gate_logits.is_contiguous()
+    assert out.shape == (T, H * V) and out.is_contiguous() and out.dtype == proj.dtype
+    assert slots.dtype == torch.int32 and slots.numel() >= S and slots.is_contiguous()
+    assert seq_runs.dtype == torch.int32 and seq_runs.shape == (S, 4) and seq_runs.is_contiguous()
+    assert seq_runs.data_ptr() % 16 == 0
+    assert state.dtype == torch.float32 and tuple(state.shape[1:]) == (H, V + 1, D) and state[0].is_contiguous()
+    assert maximum.dtype == torch.float32 and tuple(maximum.shape[1:]) == (H,) and maximum.stride(1) == 1
+    assert maximum.shape[0] == state.shape[0] and norm_w.numel() == H * V and norm_w.is_contiguous()
+    wp, wf = _param(norm_w)
+    lib = library()
+    work = torch.empty(lib.pae_matrix_memory_work_floats(T, H, D, V), dtype=torch.float32, device=proj.device)
+    _check(lib.pae_matrix_memory_step(
+        code_of(proj.dtype), proj.data_ptr(), proj.stride(0), gate.data_ptr(), gate.stride(0), gate_logits.data_ptr(), T, S,
+        seq_runs.data_ptr(), slots.data_ptr(), H, D, V, float(gate_cap), state.data_ptr(), state.stride(0),
+        maximum.data_ptr(), maximum.stride(0), wp, wf, float(norm_eps), float(floor_eps), work.data_ptr(), out.data_ptr(),
+        _stream()))
+
+
+def embedding_pairs(out: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                    tok_seq: torch.Tensor, slots: torch.Tensor, last_token: torch.Tensor, scale: float, buckets: int,
+                    mul_prev: int, mul_cur: int) -> None:
+    """out[t] = scale * table[ids[t]] + pairs[(prev * mul_prev + ids[t] * mul_cur) % buckets] as float32, `prev`
+    the token before in the same sequence (the row before in the step, or `last_token[slot]`, int32 [slots],
+    which is moved on to each sequence's last token of the step); at position 0 the row `buckets` of `pairs`.
+    A sequence's rows must be consecutive in the step and in order."""
+    _not_while_recording("embedding_pairs")
+    _gpu(out, table, pairs, ids, positions, tok_seq, slots, last_token)
+    T, H = out.shape
+    assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous() and pairs.is_contiguous()
+    assert table.dtype == pairs.dtype and table.shape[1] == H and tuple(pairs.shape) == (buckets + 1, H)
+    for t in (ids, positions, tok_seq):
+        assert t.dtype == torch.int32 and t.numel() == T and t.is_contiguous()
+    assert slots.dtype == torch.int32 and slots.is_contiguous()
+    assert last_token.dtype == torch.int32 and last_token.dim() == 1 and last_token.is_contiguous()
+    _check(library().pae_embedding_pairs(code_of(table.dtype), out.data_ptr(), table.data_ptr(), pairs.data_ptr(),
+                                         ids.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), slots.data_ptr(),
+                                         last_token.data_ptr(), T, H, table.shape[0], float(scale), int(buckets),
+                                         int(mul_prev), int(mul_cur), _stream()))
+
+
+MAX_SUM_TERMS = 4
+
+
+def sum_norm2(residual: torch.Tensor, terms, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], eps: float,
+              out1: Optional[torch.Tensor], out2: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+    """residual += sum of scale * term over `terms` (a list of (tensor, scale): [T, H] in the outputs' type or
+    float32, or float32 partial sums [P, T, H] added in order), in float32; then out1 / out2 (either may be None)
+    = residual / sqrt(mean(residual^2) + eps) * w1 / w2.  With `rows` (int32) only those rows are produced and
+    the residual is left as it is."""
+    _not_while_recording("sum_norm2")
+    outs = [o for o in (out1, out2) if o is not None]
+    _gpu(residual, w1, w2, rows, *outs, *[t for t, _ in terms])
+    H = residual.shape[-1]
+    assert residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous()
+    assert len(terms) <= MAX_SUM_TERMS
+    n = residual.shape[0] if rows is None else rows.numel()
+    dtype = outs[0].dtype if outs else torch.float32
+    for o, w in ((out1, w1), (out2, w2)):
+        if o is not None:
+            assert o.shape == (n, H) and o.is_contiguous() and o.dtype == dtype and w is not None and w.numel() == H
+    if rows is not None:
+        assert rows.dtype == torch.int32 and rows.is_contiguous()
+    count = len(terms)
+    ptrs = (c_void_p * MAX_SUM_TERMS)()
+    is_f32, parts = (c_int * MAX_SUM_TERMS)(), (c_int * MAX_SUM_TERMS)()
+    strides, scales = (c_int64 * MAX_SUM_TERMS)(), (c_float * MAX_SUM_TERMS)()
+    for j, (t, scale) in enumerate(terms):
+        assert t.is_contiguous() and tuple(t.shape[-2:]) == tuple(residual.shape)
+        if t.dim() == 3:
+            assert t.dtype == torch.float32
+        else:
+            assert t.dim() == 2 and t.dtype in (torch.float32, dtype)
+        ptrs[j], is_f32[j] = t.data_ptr(), 1 if t.dtype == torch.float32 else 0
+        parts[j], strides[j], scales[j] = (t.shape[0] if t.dim() == 3 else 1), residual.numel(), float(scale)
+    p1, f1 = _param(w1)
+    p2, f2 = _param(w2)
+    _check(library().pae_sum_norm2(code_of(dtype), residual.data_ptr(), count, ptrs, is_f32, parts, strides, scales, p1, f1,
+                                   p2, f2, float(eps), _ptr(rows), _ptr(out1), _ptr(out2), n, H, 1, _stream()))
+
+
+def project_f32(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [M, N] = a [M, K] w[N, K]^T (+ bias), summed in float32 from operands of either type: for the few
+    output features whose sums must not pass the activation type (router and gate logits)."""
+    _not_while_recording("project_f32")
+    _gpu(a, w, bias)
+    M, K = a.shape
+    assert a.dim() == 2 and a.stride(1) == 1 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == K and w.dtype == a.dtype
+    out = torch.empty((M, w.shape[0]), dtype=torch.float32, device=a.device)
+    bp, bf = _param(bias)
+    if bias is not None:
+        assert bias.numel() == w.shape[0] and bias.is_contiguous()
+    _check(library().pae_project_f32(code_of(a.dtype), out.data_ptr(), out.stride(0), a.data_ptr(), a.stride(0),
+                                     w.data_ptr(), bp, bf, M, w.shape[0], K, _stream()))
+    return out
+
+
+def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int, scale: float):
+    """(chosen int32 [T, top], weights float32 [T, top]) from router logits float32 [T, E]: scores are the softmax
+    over all experts; only experts of the `keep` best of `groups` equal groups of neighbours (a group's score is
+    its largest) can be chosen; the weights are the chosen scores times `scale`."""
+    _not_while_recording("moe_route")
+    _gpu(logits)
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    chosen = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _check(library().pae_moe_route(logits.data_ptr(), T, E, int(groups), int(keep), int(top), float(scale),
+                                   chosen.data_ptr(), weights.data_ptr(), _stream()))
+    return chosen, weights
+
+
+def moe_experts(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor, chosen: torch.Tensor,
+                weights: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """float32 [T, H]: for every token the weighted sum over its chosen experts of
+    W_down[e] (act(W_gate[e] x) * (W_up[e] x)); `gate_w`, `up_w` [E, F, H] and `down_w` [E, H, F] in x's type."""
+    _not_while_recording("moe_experts")
+    _gpu(x, gate_w, up_w, down_w, chosen, weights)
+    T, H = x.shape
+    E, F, _ = gate_w.shape
+    top = chosen.shape[1]
+    assert x.stride(1) == 1 and gate_w.shape == up_w.shape == (E, F, H) and down_w.shape == (E, H, F)
+    for w in (gate_w, up_w, down_w):
+        assert w.is_contiguous() and w.dtype == x.dtype
+    assert chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.shape[0] == T
+    assert weights.dtype == torch.float32 and weights.shape == chosen.shape and weights.is_contiguous()
+    assert activation in ACTIVATIONS
+    act = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
+    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    lib = library()
+    _check(lib.pae_moe_gate_up(code_of(x.dtype), act.data_ptr(), x.data_ptr(), x.stride(0), gate_w.data_ptr(),
+                               up_w.data_ptr(), chosen.data_ptr(), T, top, H, F, ACTIVATIONS[activation], _stream()))
+    _check(lib.pae_moe_down(code_of(x.dtype), out.data_ptr(), act.data_ptr(), down_w.data_ptr(), chosen.data_ptr(),
+                            weights.data_ptr(), T, top, H, F, _stream()))
+    return out
 
 
 def _check_bias_operands(slopes, gate, nh: int, hd: int, q: torch.Tensor):

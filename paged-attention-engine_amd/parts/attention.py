@@ -111,8 +111,8 @@ class PagedAttention(Part):
                 raise ValueError("a mask in chunks needs the chunk length (window)")
         elif not spec.own_kv:
             raise ValueError("only the convolution path knows layers without key/value tensors")
-        if not spec.plain and not spec.convolved and (spec.qkv_bias or spec.out_bias):
-            raise ValueError("an attention with value widths, caps, sinks or query/key norms takes no biases")
+        if not spec.plain and not spec.convolved and spec.out_bias:
+            raise ValueError("an attention with value widths, caps, sinks or query/key norms takes no bias on its output")
         self.position = (build_part(POSITION_ENCODINGS, "position encoding", spec.position, dtype, device)
                          if spec.position is not None else
                          POSITION_ENCODINGS["none"](None, dtype, device))
@@ -204,11 +204,11 @@ class PagedAttention(Part):
         if s.sinks:
             out[prefix + s.sink_name] = (s.num_heads,)
         if s.qkv_bias:
-            out[prefix + s.q_name + ".bias"] = (s.num_heads * s.head_dim,)
-            out[prefix + s.k_name + ".bias"] = (s.num_kv_heads * s.head_dim,)
-            out[prefix + s.v_name + ".bias"] = (s.num_kv_heads * s.head_dim,)
+            out[prefix + s.q_name + s.bias_suffix] = (s.num_heads * s.head_dim,)
+            out[prefix + s.k_name + s.bias_suffix] = (s.num_kv_heads * s.head_dim,)
+            out[prefix + s.v_name + s.bias_suffix] = (s.num_kv_heads * s.v_dim,)
         if s.out_bias:
-            out[prefix + s.o_name + ".bias"] = (s.hidden_size,)
+            out[prefix + s.o_name + s.bias_suffix] = (s.hidden_size,)
         return out
 
     def _bind_convolved(self, prefix, weights):
@@ -239,11 +239,11 @@ class PagedAttention(Part):
             return self._bind_convolved(prefix, weights)
         names = (s.q_name, s.k_name, s.v_name)
         w = torch.cat([weights[prefix + n + s.weight_suffix] for n in names], dim=0)
-        b = (torch.cat([weights[prefix + n + ".bias"] for n in names], dim=0) if s.qkv_bias else None)
+        b = (torch.cat([weights[prefix + n + s.bias_suffix] for n in names], dim=0) if s.qkv_bias else None)
         self.qkv = Linear(self.matrix(w), None if b is None else self.vector(b))
         nq = s.num_heads * s.head_dim
         self.q_only = Linear(self.qkv.weight[:nq], None if b is None else self.qkv.bias[:nq])
-        ob = weights[prefix + s.o_name + ".bias"] if s.out_bias else None
+        ob = weights[prefix + s.o_name + s.bias_suffix] if s.out_bias else None
         self.out = Linear(self.matrix(weights[prefix + s.o_name + s.weight_suffix]), None if ob is None else self.vector(ob))
         self.q_norm = self.k_norm = self.sinks = None
         if s.qk_norm:

@@ -95,6 +95,13 @@ class ResidualStream:
         self.sum_weights: Optional[torch.Tensor] = None
 
 
+class BranchTerms(list):
+    """What a block's branches leave pending on the stream when there are several of them: a list of
+    (tensor, factor), each tensor [T, H] in the activation type or float32, or float32 partial sums
+    [P, T, H]; the norm that reads the stream next adds factor * tensor for each, in order, in float32.
+    A mixer that is several mixers side by side may return one as its output."""
+
+
 class StreamJoin:
     """How a pending branch output joins a stream that is kept in several copies: every copy t becomes
     sum_s mix[s, t] x_s + out[t] * (scale * y), `scale` one factor per feature (None: none).  `mix`

@@ -7,8 +7,8 @@ left pending on the stream and added by the next norm, in float32.
 
 from __future__ import annotations
 
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BranchSink, Part, ResidualStream, ScaleShape, StreamJoin,
-                   build_part, plain_rows, register_block)
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BranchSink, BranchTerms, Part, ResidualStream, ScaleShape,
+                   StreamJoin, build_part, plain_rows, register_block)
 
 
 @register_block("prenorm")
@@ -253,6 +253,68 @@ class HyperBlock:
         if self.feed_forward is not None:
             x = self.feed_forward_norm.forward_copies(stream, self.reads[1])
             stream.pending, stream.join = self.feed_forward.forward(ctx, x), self.joins[1]
+
+
+@register_block("parallel")
+class ParallelBlock:
+    """Both branches read the same stream, each through a norm of its own:
+    x <- x + mixer(norm1(x)) + feed_forward(norm2(x)).  A layer whose spec names no feed-forward has the
+    mixer alone.  The branches' outputs stay pending on the stream as `BranchTerms`; the kernel that
+    norms the stream for the next block (or the model's last norm) adds them into the float32 residual
+    first, and forms both of this block's norms from one pass over the row."""
+
+    def __init__(self, layer_spec, dtype, device):
+        self.spec = layer_spec
+        self.first_norm = build_part(NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.mixer = build_part(MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.second_norm = self.feed_forward = None
+        if layer_spec.feed_forward is not None:
+            self.second_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
+            self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+        for norm in (self.first_norm, self.second_norm):
+            if norm is not None and not hasattr(norm, "forward_pair"):
+                raise ValueError(f"the norm '{norm.spec.kind}' cannot share a pass over the stream (no forward_pair)")
+
+    def _named(self):
+        s = self.spec
+        out = [(self.first_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix)]
+        if self.feed_forward is not None:
+            out += [(self.second_norm, s.prefix + s.feed_forward_norm_prefix),
+                    (self.feed_forward, s.prefix + s.feed_forward_prefix)]
+        return out
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for part, _ in self._named())
+
+    @property
+    def graph_max_rows(self):
+        limits = [part.graph_max_rows for part, _ in self._named() if part.graph_max_rows is not None]
+        return min(limits) if limits else None
+
+    def parts(self):
+        return [part for part, _ in self._named()]
+
+    def tensors(self):
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        return out
+
+    def bind(self, weights):
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+
+    def forward(self, ctx, stream: ResidualStream) -> None:
+        ctx.sink = None
+        x1, x2 = self.first_norm.forward_pair(stream, self.second_norm)
+        terms = BranchTerms()
+        for y in (self.mixer.forward(ctx, x1), self.feed_forward.forward(ctx, x2) if self.feed_forward is not None else None):
+            if isinstance(y, BranchTerms):
+                terms.extend(y)
+            elif y is not None:
+                terms.append((y, 1.0))
+        stream.pending = terms
 
 
 def build_block(layer_spec, dtype, device):

@@ -10,6 +10,11 @@ value W_uv_j c; query and shared key part are rotated by position; the score is
 over the keys the mask lets through (a sliding window, chunks, or every earlier key), an ordinary
 softmax, and W_o on the concatenated heads.
 
+For designs that have them: a learned sink per head that joins the softmax's denominator as exp(sink), without
+a key or a value and not scaled (`sinks`); no rotated part at all (`rope_dim` 0); and layers without a down
+projection that read the rows an earlier layer cached, with their own W_uk, W_uv, queries and mask (`own_kv` False:
+the stop borrows that layer's pages).
+
 What the cache holds of a token is c and the rotated part, one row of kv_rank + rope_dim whatever the number
 of heads (`paged_spec`: one tensor "latent" [PAGE][kv_rank + rope_dim]).  The heads' keys and values
 are never formed: since q_nope . (W_uk_j c) = (W_uk_j^T q_nope) . c, the query is folded into latent
@@ -65,6 +70,8 @@ class LatentAttention(Part):
             raise ValueError(f"mask '{spec.mask}' is not known (known: window, chunk)")
         if spec.mask == "chunk" and not spec.window:
             raise ValueError("a mask in chunks needs the chunk length (window)")
+        if not spec.own_kv and spec.rope_dim:
+            raise ValueError("a latent layer that reads another layer's rows has no rotated part")
         rotated = getattr(spec.position, "rotary_dim", 0) if spec.position is not None else 0
         if rotated > spec.rope_dim:
             raise ValueError(f"{rotated} rotated features of a rotated part of {spec.rope_dim}")
@@ -89,7 +96,7 @@ class LatentAttention(Part):
     @property
     def matrix_cores(self) -> bool:
         """Whether the attention runs on the matrix cores (then the pages also hold the latents transposed)."""
-        return K.latent_attn_supported(self.dtype, self.row_width, self.spec.kv_rank)
+        return not self.spec.sinks and K.latent_attn_supported(self.dtype, self.row_width, self.spec.kv_rank)
 
     def paged_spec(self):
         s = self.spec
@@ -108,19 +115,26 @@ class LatentAttention(Part):
     def tensors(self, prefix):
         s = self.spec
         sfx = s.weight_suffix
-        return {prefix + s.q_name + sfx: (s.num_heads * (s.nope_dim + s.rope_dim), s.hidden_size),
-                prefix + s.down_name + sfx: (self.row_width, s.hidden_size),
-                prefix + s.down_norm_name: ScaleShape((s.kv_rank,)),
-                prefix + s.up_k_name + sfx: (s.num_heads * s.nope_dim, s.kv_rank),
-                prefix + s.up_v_name + sfx: (s.num_heads * s.value_dim, s.kv_rank),
-                prefix + s.o_name + sfx: (s.hidden_size, s.num_heads * s.value_dim)}
+        out = {prefix + s.q_name + sfx: (s.num_heads * (s.nope_dim + s.rope_dim), s.hidden_size),
+               prefix + s.up_k_name + sfx: (s.num_heads * s.nope_dim, s.kv_rank),
+               prefix + s.up_v_name + sfx: (s.num_heads * s.value_dim, s.kv_rank),
+               prefix + s.o_name + sfx: (s.hidden_size, s.num_heads * s.value_dim)}
+        if s.own_kv:
+            out[prefix + s.down_name + sfx] = (self.row_width, s.hidden_size)
+            out[prefix + s.down_norm_name] = ScaleShape((s.kv_rank,))
+        if s.sinks:
+            out[prefix + s.sink_name] = (s.num_heads,)
+        return out
 
     def bind(self, prefix, weights):
         s = self.spec
         sfx = s.weight_suffix
-        self.proj = Linear(self.matrix(torch.cat([weights[prefix + s.q_name + sfx], weights[prefix + s.down_name + sfx]],
-                                                 dim=0)))
-        self.down_norm = self.vector(weights[prefix + s.down_norm_name])
+        projected = [weights[prefix + s.q_name + sfx]] + ([weights[prefix + s.down_name + sfx]] if s.own_kv else [])
+        self.proj = Linear(self.matrix(torch.cat(projected, dim=0)))
+        self.down_norm = self.vector(weights[prefix + s.down_norm_name]) if s.own_kv else None
+        # sinks enter the softmax, which is float32
+        self.sinks = (weights[prefix + s.sink_name].to(device=self.device, dtype=torch.float32).contiguous()
+                      if s.sinks else None)
         up_k = weights[prefix + s.up_k_name + sfx].view(s.num_heads, s.nope_dim, s.kv_rank)
         # the fold q_nope -> W_uk^T q_nope is a product with W_uk^T as its [out, in] matrix, head by head
         self.up_k_t = self.matrix(up_k.transpose(1, 2))
@@ -129,8 +143,8 @@ class LatentAttention(Part):
 
     def forward(self, ctx, x):
         s = self.spec
-        if not ctx.writes_cache:
-            raise ValueError("a latent attention layer keeps pages of its own")
+        if s.own_kv != ctx.writes_cache:
+            raise ValueError("a latent layer with a down projection writes its own pages, one without reads another stop's")
         x = plain_rows(x)
         T, H, C, R, D, V = x.shape[0], s.num_heads, s.kv_rank, s.rope_dim, s.nope_dim, s.value_dim
         pages = ctx.cache.pages_of(ctx.cache_entry)
@@ -139,12 +153,13 @@ class LatentAttention(Part):
         proj = self.proj(x)
         rot, cos_sin = self.position.rotary_table(ctx)
         q_full = torch.empty((T, H * (C + R)), dtype=proj.dtype, device=proj.device)
-        K.latent_prepare(proj, q_full, H, D, R, rot, bool(getattr(self.position, "interleaved", False)), C,
-                         self.down_norm, s.norm_eps, cos_sin, ctx.positions, ctx.tok_seq, table, latent, latent_t)
+        if s.own_kv:
+            K.latent_prepare(proj, q_full, H, D, R, rot, bool(getattr(self.position, "interleaved", False)), C,
+                             self.down_norm, s.norm_eps, cos_sin, ctx.positions, ctx.tok_seq, table, latent, latent_t)
         K.heads_product(q_full.view(T, H, C + R)[:, :, :C], proj[:, :H * (D + R)].view(T, H, D + R)[:, :, :D], self.up_k_t)
         summed = torch.empty((T, H * C), dtype=proj.dtype, device=proj.device)
         key = self.step_lists_key(ctx.cache.block_size)
-        if key is not None:
+        if key is not None and latent_t is not None:
             tiles = ctx.memo[key]
             for name, column_tiles in (("single", 1), ("runs", 2)):
                 if tiles[name].numel():
@@ -152,7 +167,7 @@ class LatentAttention(Part):
                                   s.scale, s.window or 0, s.mask == "chunk")
         else:
             K.paged_attention_masked(summed, q_full, latent, None, ctx.positions, ctx.tok_seq, table, H, 1, C + R, C, s.scale,
-                                     s.window or 0, s.mask == "chunk")
+                                     s.window or 0, s.mask == "chunk", sinks=self.sinks)
         heads = torch.empty((T, H * V), dtype=proj.dtype, device=proj.device)
         K.heads_product(heads.view(T, H, V), summed.view(T, H, C), self.up_v)
         return self.out.branch(heads, ctx.sink)

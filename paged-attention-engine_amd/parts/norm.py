@@ -13,17 +13,24 @@ from typing import Optional
 import torch
 
 from ..kernels import lib as K
-from .base import OwedRows, Part, ResidualStream, ScaleShape, register_norm
+from .base import BranchTerms, OwedRows, Part, ResidualStream, ScaleShape, register_norm
 
 
 @register_norm("rmsnorm")
 class RMSNorm(Part):
     graph_safe = True
     def tensors(self, prefix):
-        return {prefix + self.spec.weight_name: ScaleShape((self.spec.size,))}
+        # a weight that is stored minus an offset lies around zero like any other tensor
+        shape = (self.spec.size,)
+        return {prefix + self.spec.weight_name: shape if self.spec.weight_offset else ScaleShape(shape)}
 
     def bind(self, prefix, weights):
-        self.weight = self.vector(weights[prefix + self.spec.weight_name])
+        stored = weights[prefix + self.spec.weight_name]
+        if self.spec.weight_offset:
+            # offset + w is formed in float32 and stays so: rounded to the storage type it would lose w's last bits
+            self.weight = (stored.to(device=self.device, dtype=torch.float32) + float(self.spec.weight_offset)).contiguous()
+        else:
+            self.weight = self.vector(stored)
 
     def folded_for(self, rows: int):
         """(weight, eps) if, in a step of `rows` rows, whatever writes the residual before this norm
@@ -45,6 +52,8 @@ class RMSNorm(Part):
         and prepared this norm's rows, they are returned as they are (`OwedRows`): no kernel runs."""
         if stream.copies > 1 or stream.join is not None:
             return self.forward_copies(stream, stream.sum_weights, rows)
+        if isinstance(stream.pending, BranchTerms):
+            return self.forward_pair(stream, None, rows)[0]
         if stream.owed is not None:
             owed, mine = stream.owed, stream.owed_to is self
             if rows is None:
@@ -58,6 +67,25 @@ class RMSNorm(Part):
         if rows is None:
             stream.pending = None
         return out
+
+    def forward_pair(self, stream: ResidualStream, other: Optional["RMSNorm"], rows: Optional[torch.Tensor] = None):
+        """For blocks whose branches read the same stream: the pending branches (a tensor, or `BranchTerms`)
+        join the residual, and the new residual is normed by this norm and by `other` (None: by this one
+        alone) in one kernel.  Returns both results.  With `rows` only those rows, and the stream stays as it is."""
+        if stream.owed is not None or stream.copies > 1:
+            raise ValueError("a norm for two branches reads a plain stream with nothing prepared for another norm")
+        pending = stream.pending
+        terms = pending if isinstance(pending, BranchTerms) else BranchTerms([] if pending is None else [(pending, 1.0)])
+        n = stream.residual.shape[0] if rows is None else rows.numel()
+        new = lambda: torch.empty((n, self.spec.size), dtype=self.dtype, device=stream.residual.device)
+        out1, out2 = new(), (new() if other is not None else None)
+        if other is not None and other.spec.eps != self.spec.eps:
+            raise ValueError("two norms of one stream in one kernel share their eps")
+        K.sum_norm2(stream.residual, terms, self.weight, other.weight if other is not None else None, self.spec.eps,
+                    out1, out2, rows)
+        if rows is None:
+            stream.pending = None
+        return out1, out2
 
     def forward_copies(self, stream: ResidualStream, read_weights: torch.Tensor,
                        rows: Optional[torch.Tensor] = None):

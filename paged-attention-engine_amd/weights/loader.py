@@ -74,6 +74,12 @@ def _open_shards(model_dir: str) -> Dict[str, SafetensorsFile]:
     return by_name
 
 
+def stored_shapes(model_dir: str) -> Dict[str, Tuple[int, ...]]:
+    """name -> shape of every tensor the folder's checkpoint holds, read from the files' headers alone: for
+    architectures some of whose sizes stand in no config key but in a tensor's shape."""
+    return {name: tuple(shard.shape(name)) for name, shard in _open_shards(model_dir).items()}
+
+
 def _keep_precision(t: torch.Tensor) -> torch.Tensor:
     if t.dtype in (torch.bfloat16, torch.float32, torch.int32):
         return t
