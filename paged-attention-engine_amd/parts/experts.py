@@ -40,6 +40,9 @@ class Experts(Part):
                              f"{spec.groups_kept * (spec.num_experts // spec.groups)} can be")
         if spec.num_experts > 1024:
             raise ValueError(f"{spec.num_experts} experts: the routing kernel takes up to 1024")
+        # for comparing a model with another implementation: called after every routing with (chosen, weights);
+        # a step with a tap that reads them on the host cannot be recorded as a graph
+        self.routing_tap = None
 
     def _expert(self, prefix: str, index: int, name: str) -> str:
         s = self.spec
@@ -73,4 +76,6 @@ class Experts(Part):
         x = plain_rows(x)
         logits = K.project_f32(x, self.router)
         chosen, weights = K.moe_route(logits, s.groups, s.groups_kept, s.top, s.route_scale)
+        if self.routing_tap is not None:
+            self.routing_tap(chosen, weights)
         return K.moe_experts(x, self.gate, self.up, self.down, chosen, weights, s.activation)

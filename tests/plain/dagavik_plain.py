@@ -173,8 +173,9 @@ def matrix_memory(W: dict, prefix: str, m: dict, h: torch.Tensor, eps: float, dt
     q = product(h, get("q")).view(T, H, D) * D ** -0.5
     k = product(h, get("k")).view(T, H, D)
     v = product(h, get("v")).view(T, H, V)
-    log_in = soft_cap(product(h, get("i")) + get("i.b"), cap)
-    log_keep = log_sigmoid(soft_cap(product(h, get("f")) + get("f.b"), cap))
+    # the gates' logarithms add up over a sequence: their sums do not pass the storage type
+    log_in = soft_cap(stored(h) @ get("i").T + get("i.b"), cap)
+    log_keep = log_sigmoid(soft_cap(stored(h) @ get("f").T + get("f.b"), cap))
     o = matrix_memory_recurrence(q, k, v, log_in, log_keep)
     o = rms(o, eps).reshape(T, H * V) * get("norm") * sigmoid(product(h, get("g")))
     return product(o, get("o"))
@@ -258,8 +259,11 @@ def channel_delta(W: dict, prefix: str, m: dict, h: torch.Tensor, eps: float, dt
 # --------------------------------------------------------------------------- feed-forward
 
 
-def route(z: torch.Tensor, router: dict):
-    """z [T, E] router logits -> (chosen experts [T, top], their weights [T, top])."""
+def route(z: torch.Tensor, router: dict, margins=None):
+    """z [T, E] router logits -> (chosen experts [T, top], their weights [T, top]).  `margins`, a list,
+    receives [T]: how far, in units of the logits, each token's choice is from another one (the
+    smaller of the gaps between the last group kept and the first one dropped, and between the last
+    expert chosen and the first one passed over)."""
     E, top = z.shape[1], int(router["top"])
     groups = router.get("groups") or {"count": 1, "keep": 1}
     count, keep = int(groups["count"]), int(groups["keep"])
@@ -270,6 +274,15 @@ def route(z: torch.Tensor, router: dict):
     allowed.scatter_(1, kept, True)
     masked = torch.where(allowed.repeat_interleave(E // count, dim=1), s, torch.full_like(s, -1.0))
     chosen = masked.topk(top, dim=-1).indices
+    if margins is not None:
+        gap = torch.full((z.shape[0],), float("inf"), dtype=z.dtype)
+        if keep < count:
+            ranked = torch.log(best).sort(dim=-1, descending=True).values
+            gap = ranked[:, keep - 1] - ranked[:, keep]
+        if top < keep * (E // count):
+            ranked = torch.log(masked.clamp_min(1e-300)).sort(dim=-1, descending=True).values
+            gap = torch.minimum(gap, ranked[:, top - 1] - ranked[:, top])
+        margins.append(gap)
     return chosen, s.gather(1, chosen) * float(router["scale"])
 
 
@@ -278,9 +291,15 @@ def expert(W: dict, prefix: str, h: torch.Tensor, dtype) -> torch.Tensor:
     return product(act, W[prefix + "down"].to(dtype))
 
 
-def mixture(W: dict, prefix: str, mlp: dict, h: torch.Tensor, dtype) -> torch.Tensor:
+def mixture(W: dict, prefix: str, mlp: dict, h: torch.Tensor, dtype, margins=None, forced=None) -> torch.Tensor:
+    """`forced` [T, top]: experts to use instead of the ones `route` chooses (their weights are still this
+    function's own scores), for comparing with an implementation in reduced precision, where a choice
+    between two nearly equal scores may fall the other way."""
     z = stored(h) @ W[prefix + "router"].to(dtype).T
-    chosen, weights = route(z, mlp["router"])
+    chosen, weights = route(z, mlp["router"], margins)
+    if forced is not None:
+        chosen = torch.as_tensor(forced, dtype=torch.long)
+        weights = torch.softmax(z, dim=-1).gather(1, chosen) * float(mlp["router"]["scale"])
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weights[t]):
@@ -291,8 +310,10 @@ def mixture(W: dict, prefix: str, mlp: dict, h: torch.Tensor, dtype) -> torch.Te
 # --------------------------------------------------------------------------- the model
 
 
-def forward(W: dict, cfg: dict, tokens, dtype=torch.float64, taps=None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence.  `taps`, a list, receives the stream after every layer."""
+def forward(W: dict, cfg: dict, tokens, dtype=torch.float64, taps=None, margins=None, routing=None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence.  `taps`, a list, receives the stream after every layer;
+    `margins`, a list, every feed-forward's routing margins [T] (see `route`); `routing` {layer: experts
+    [T, top]} forces those layers' choices (see `mixture`)."""
     eps = float(cfg["norm"]["eps"])
     x = embed(W, cfg, tokens, dtype)
     latents = {}
@@ -311,15 +332,18 @@ def forward(W: dict, cfg: dict, tokens, dtype=torch.float64, taps=None) -> torch
         else:
             raise ValueError(f"unknown layer type {layer['type']!r}")
         if layer.get("mlp") is not None:
-            y = y + mixture(W, at + "mlp.", layer["mlp"], offset_norm(x, W[at + "norm2"].to(dtype), eps), dtype)
+            y = y + mixture(W, at + "mlp.", layer["mlp"], offset_norm(x, W[at + "norm2"].to(dtype), eps), dtype, margins,
+                            None if routing is None else routing.get(i))
         x = x + y
         if taps is not None:
             taps.append(x.clone())
     return product(offset_norm(x, W["final.norm"].to(dtype), eps), W["head"].to(dtype))
 
 
-def greedy_generate(W: dict, cfg: dict, prompt, count: int, dtype=torch.float64) -> list:
-    tokens = list(prompt)
+def greedy_generate(W: dict, cfg: dict, prompt, count: int, dtype=torch.float64):
+    """(the `count` tokens that follow `prompt` greedily, the logits each was chosen from [count, vocab])."""
+    tokens, rows = list(prompt), []
     for _ in range(count):
-        tokens.append(int(forward(W, cfg, tokens, dtype)[-1].argmax()))
-    return tokens[len(prompt):]
+        rows.append(forward(W, cfg, tokens, dtype)[-1])
+        tokens.append(int(rows[-1].argmax()))
+    return tokens[len(prompt):], torch.stack(rows)
