@@ -104,10 +104,44 @@ def ritalorn_shape(shape: dict, layers: int) -> dict:
             "norm": {"eps": shape["rms_norm_eps"]}, "streams": 4, "logit_softcap": 30.0, "layers": out}
 
 
+def dagavik_shape(shape: dict, layers: int) -> dict:
+    """A Dagavik configuration with the layer sizes of the Qwen2.5 shape `shape`: the same width, head counts and
+    head size in the attention half of its parallel layers (values as wide as keys, half of each head rotated, a
+    window of 2,048) beside a matrix memory with as many heads of the same size; latent attention in every
+    fourth layer from the second on (as many heads, a latent of four head sizes), the later ones reading the
+    first one's rows; gated delta layers with a decay per key channel (half as many query/key heads,
+    convolutions of four taps, narrow products of half a head size); a feed-forward of 32 experts in four
+    groups of which two are kept, four experts a token, each a quarter of the shape's feed-forward wide, so
+    that a token's feed-forward does the arithmetic of the dense one; the same vocabulary; a bigram table of
+    65,521 rows.  Layers in turn: parallel, latent, delta, delta."""
+    heads, kv, hd = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    mlp = {"kind": "moe", "expert": {"ff": shape["intermediate_size"] // 4 // 8 * 8},
+           "router": {"experts": 32, "top": 4, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    parallel = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 2048},
+                 "rot": {"base": float(shape["rope_theta"]), "dims": hd // 2}},
+        "right": {"heads": heads, "dim": hd, "vdim": hd, "gate_cap": 15.0}, "left_scale": 0.7, "right_scale": 0.7}}
+    delta = {"type": "channel_delta", "mlp": mlp,
+             "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": hd, "vdim": hd, "conv": 4,
+                       "decay_rank": hd // 2, "gate_rank": hd // 2}}
+    out = []
+    for i in range(layers):
+        if i % 4 == 1:
+            mixer = {"heads": heads, "dim": hd, "vdim": hd, "kv_rank": 4 * hd, "scale": hd ** -0.5}
+            if i > 1:
+                mixer["kv_from"] = 1
+            out.append({"type": "latent_attention", "mlp": mlp, "mixer": mixer})
+        else:
+            out.append(parallel if i % 4 == 0 else delta)
+    return {"architecture": "Dagavik", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
+            "norm": {"eps": shape["rms_norm_eps"]},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": out}
+
+
 def design_run(args, shape: dict) -> int:
-    """`--design danonex|ritalorn`: decode steps (batch 1, 8, 64 at the context asked for) and prefills of
+    """`--design danonex|ritalorn|dagavik`: decode steps (batch 1, 8, 64 at the context asked for) and prefills of
     2,048 and 8,192 tokens of a model of that design with the shape's layer sizes, and beside each the same
-    measurement of the Qwen2.5 shape (and, for ritalorn, of the Danonex shape) with the same number of
+    measurement of the Qwen2.5 shape (and, for ritalorn and dagavik, of the Danonex shape) with the same number of
     layers.  One JSON line."""
     import torch
 
@@ -117,7 +151,11 @@ def design_run(args, shape: dict) -> int:
                         f"prefill tok/s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "context": args.ctx,
               "data": "synthetic: seeded uniform token ids, random weights N(0, 0.02)", "designs": {}}
-    if args.design == "ritalorn":
+    if args.design == "dagavik":
+        configs = {"dagavik": dagavik_shape(shape, layers)}
+        if not args.alone:
+            configs.update({"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)})
+    elif args.design == "ritalorn":
         configs = {"ritalorn": ritalorn_shape(shape, layers)}
         if not args.alone:
             configs.update({"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)})
@@ -371,11 +409,11 @@ def main() -> int:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
-    parser.add_argument("--design", choices=("qwen2", "danonex", "ritalorn"), default="qwen2",
-                        help="danonex, ritalorn: a model of that design with the shape's layer sizes (8 layers unless "
-                             "--layers says otherwise) beside the Qwen2.5 shape (ritalorn: and the Danonex shape) with "
+    parser.add_argument("--design", choices=("qwen2", "danonex", "ritalorn", "dagavik"), default="qwen2",
+                        help="danonex, ritalorn, dagavik: a model of that design with the shape's layer sizes (8 layers unless "
+                             "--layers says otherwise) beside the Qwen2.5 shape (ritalorn, dagavik: and the Danonex shape) with "
                              "as many layers: decode at batch 1, 8, 64 and prefills of 2,048 and 8,192 tokens")
-    parser.add_argument("--alone", action="store_true", help="with --design ritalorn: that design only (for profiles)")
+    parser.add_argument("--alone", action="store_true", help="with --design ritalorn or dagavik: that design only (for profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (run with --gpus 1)")
@@ -386,7 +424,7 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
     shape = QWEN25_1P5B if args.model == "1.5b" else OTHER_SHAPES[args.model]
-    if args.design in ("danonex", "ritalorn"):
+    if args.design in ("danonex", "ritalorn", "dagavik"):
         try:
             return design_run(args, shape)
         except (Refused, Unresolved) as err:

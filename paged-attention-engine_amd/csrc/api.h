@@ -96,7 +96,7 @@ int pae_latent_attn_columns(int H, int ct);
 int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* latent,
                          const void* latent_t, const int* tiles, int num_tiles, int ct, const int* positions,
                          const int* block_tables, int max_blocks, int bs, int H, int kd, int C, float scale, int window,
-                         int chunked, float* part_acc, float* part_ml, hipStream_t stream);
+                         int chunked, float* part_acc, float* part_ml, const float* sinks, hipStream_t stream);
 int pae_latent_attn_split();
 // rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
 int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
@@ -141,6 +141,12 @@ int pae_moe_route(const float* logits, int num_tokens, int experts, int groups, 
                   int* chosen, float* weights, hipStream_t stream);
 int pae_moe_gate_up(int dtype, void* act, const void* x, int64_t ldx, const void* gate_w, const void* up_w,
                     const int* chosen, int num_tokens, int top, int hidden, int inter, int act_kind, hipStream_t stream);
+int pae_moe_tile_rows(int pairs);
+int pae_moe_max_tiles(int pairs, int experts);
+int pae_moe_tiles_supported(int hidden, int inter);
+int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const void* gate_w, const void* up_w, const void* down_w,
+                          const int* chosen, const float* weights, int num_tokens, int top, int experts, int hidden,
+                          int inter, int act_kind, int* order, int* tiles, void* act, hipStream_t stream);
 int pae_moe_down(int dtype, float* out, const void* act, const void* down_w, const int* chosen, const float* weights,
                  int num_tokens, int top, int hidden, int inter, hipStream_t stream);
 int pae_attn_decode_split();

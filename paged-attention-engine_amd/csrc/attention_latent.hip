@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
     const bf16_t* __restrict__ latent, const bf16_t* __restrict__ latent_t, const int4* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int H, int C,
     float scale_log2, int window, int chunked, int num_splits, int split_len, float* __restrict__ part_acc,
-    float* __restrict__ part_ml) {
+    float* __restrict__ part_ml, const float* __restrict__ sinks) {
   extern __shared__ float s_buf[];  // [3 or 1][CT][VS / 4 + 2][64]
   constexpr int ROWS = VS / 4 + 2;
   const int lane = threadIdx.x % PAE_WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE);
@@ -203,6 +203,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
       }
       continue;
     }
+    // a sink joins the denominator as exp(sink), unscaled, with no key and no value
+    if (sinks) sum += exp2f(sinks[head[ct]] * LOG2E - m[ct]);
     const float inv = 1.0f / sum;
     bf16_t* o = out + (int64_t)tok[ct] * out_stride + (int64_t)head[ct] * C + (int64_t)slice * VS;
 #pragma unroll
@@ -220,7 +222,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
 __global__ void latent_attn_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_acc,
                                          const float* __restrict__ part_ml, const int4* __restrict__ tiles,
                                          const int* __restrict__ positions, int H, int C, int window, int chunked,
-                                         int num_splits, int split_len) {
+                                         int num_splits, int split_len, const float* __restrict__ sinks) {
   const int4 tile = tiles[blockIdx.x];
   const int head = blockIdx.y, tok = tile.y;
   const int pos = positions[tok];
@@ -239,6 +241,7 @@ __global__ void latent_attn_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
     l = l * f_old + ls * f;
     m = m_new;
   }
+  if (sinks) l += exp2f(sinks[head] * LOG2E - m);
   const float inv = 1.0f / l;
   s16x4 w;
 #pragma unroll
@@ -258,7 +261,7 @@ static size_t latent_lds_bytes(int ct, int vs) {  // three wavefronts' states if
 // Key widths (latent + rotated part) the kernel is built for; the value slice is the largest of 128, 64, 32 that divides C.
 extern "C" int pae_latent_attn_supported(int kd, int C, int bs) {
   const bool kd_ok = kd == 64 || kd == 96 || kd == 128 || kd == 160 || kd == 192 || kd == 256 || kd == 288 || kd == 320 ||
-                     kd == 384 || kd == 576;
+                     kd == 384 || kd == 512 || kd == 576;
   return kd_ok && C % 32 == 0 && C > 0 && C <= kd && bs >= 16 && bs % 16 == 0;
 }
 
@@ -271,7 +274,8 @@ extern "C" int pae_latent_attn_columns(int H, int ct) {  // tokens a tile of 16 
 extern "C" int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* latent,
                                     const void* latent_t, const int* tiles, int num_tiles, int ct, const int* positions,
                                     const int* block_tables, int max_blocks, int bs, int H, int kd, int C, float scale,
-                                    int window, int chunked, float* part_acc, float* part_ml, hipStream_t stream) {
+                                    int window, int chunked, float* part_acc, float* part_ml, const float* sinks,
+                                    hipStream_t stream) {
   PAE_REQUIRE(pae_latent_attn_supported(kd, C, bs), "latent attention: row width %d / latent %d / page size %d are not built", kd, C,
               bs);
   PAE_REQUIRE(H > 0 && H <= 16 * 65535 && max_blocks > 0 && window >= 0, "latent attention: bad sizes H=%d max_blocks=%d window=%d",
@@ -297,7 +301,7 @@ extern "C" int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q
   latent_attn_kernel<KD, VS, CT><<<grid, 256, latent_lds_bytes(CT, VS), stream>>>(                                       \
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)latent, (const bf16_t*)latent_t,             \
       (const int4*)tiles, positions, block_tables, max_blocks, bs, H, C, scale_log2, window, chunked, num_splits,       \
-      LATENT_SPLIT, part_acc, part_ml)
+      LATENT_SPLIT, part_acc, part_ml, sinks)
 #define LAT_BY_CT(KD, VS)        \
   if (ct == 1) {                 \
     LAT_LAUNCH(KD, VS, 1);       \
@@ -322,6 +326,7 @@ extern "C" int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q
     case 288: LAT_BY_VS(288); break;
     case 320: LAT_BY_VS(320); break;
     case 384: LAT_BY_VS(384); break;
+    case 512: LAT_BY_VS(512); break;
     case 576: LAT_BY_VS(576); break;
     default: return pae_fail("latent attention: row width %d is not built", kd);
   }
@@ -332,7 +337,7 @@ extern "C" int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q
     const int threads = (C / 4 + PAE_WAVE - 1) / PAE_WAVE * PAE_WAVE;
     latent_attn_merge_kernel<<<dim3(num_tiles, H), threads, 0, stream>>>((bf16_t*)out, out_stride, part_acc, part_ml,
                                                                        (const int4*)tiles, positions, H, C, window, chunked,
-                                                                       num_splits, LATENT_SPLIT);
+                                                                       num_splits, LATENT_SPLIT, sinks);
   }
   return pae_check_launch("latent_attn");
 }

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ act, c
     }
     gs = wave_sum(gs);
     us = wave_sum(us);
-    // both sums pass the activation type, as the products of the dense feed-forwards do
+    // the gate is applied to the float32 sums and the product rounded once
     if (lane == 0) act[pair * inter + f] = from_f32<T>(act_of(gs, act_kind) * us);
   }
 }
@@ -215,4 +215,179 @@ extern "C" int pae_moe_down(int dtype, float* out, const void* act, const void* 
   else
     return pae_fail("experts: unknown dtype code %d", dtype);
   return pae_check_launch("moe_down");
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The experts on the matrix cores (bfloat16, widths in multiples of 32).  The (token, expert) pairs of a step are
+// sorted by expert on the device, and every expert's pairs are cut into tiles of up to 16 MT rows; a workgroup takes one
+// tile and 64 output features, its four wavefronts 16 features each, so an expert's weights are streamed once per
+// tile: once in all for a step of a few tokens, and once per 16 MT of an expert's tokens in a prompt.  Which tile a
+// pair falls into changes nothing of its sums (k ascends in steps of 32 for every row by itself), so a token's
+// result does not depend on the batch.
+//
+//   moe_sort            counts, offsets and tiles by expert (one workgroup; the order of an expert's pairs among
+//                       themselves is whatever the counters' turn gives, and does not matter)
+//   moe_tiles_gate_up   act(W_gate x) * (W_up x) for a tile's rows, rounded, to rows in sorted order
+//   moe_tiles_down      weight * W_down act for a tile's rows, float32, to y[chosen place][token]: the `top` places
+//                       of a token are float32 partial sums that the stream's next norm adds in order
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ chosen, int pairs, int experts, int tile_rows,
+                                                        int* __restrict__ order, int4* __restrict__ tiles, int max_tiles) {
+  extern __shared__ int sorted_lds[];  // [experts] counts, starts, cursors, first tiles; [1] tiles in all
+  int* count = sorted_lds;
+  int* start = count + experts;
+  int* cursor = start + experts;
+  int* first_tile = cursor + experts;
+  int* total = first_tile + experts;
+  for (int e = threadIdx.x; e < experts; e += 1024) count[e] = cursor[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += 1024) atomicAdd(&count[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int rows = 0, tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      start[e] = rows;
+      first_tile[e] = tile;
+      rows += count[e];
+      tile += (count[e] + tile_rows - 1) / tile_rows;
+    }
+    *total = tile;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += 1024) {
+    const int e = chosen[p];
+    order[start[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+  for (int e = threadIdx.x; e < experts; e += 1024)
+    for (int j = 0; j * tile_rows < count[e]; ++j)
+      tiles[first_tile[e] + j] = make_int4(e, start[e] + j * tile_rows, min(tile_rows, count[e] - j * tile_rows), 0);
+  for (int i = *total + threadIdx.x; i < max_tiles; i += 1024) tiles[i] = make_int4(0, 0, 0, 0);
+}
+
+template <int MT>
+__global__ __launch_bounds__(256) void moe_tiles_gate_up_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ x,
+                                                                int64_t ldx, const bf16_t* __restrict__ gate_w,
+                                                                const bf16_t* __restrict__ up_w, const int* __restrict__ order,
+                                                                const int4* __restrict__ tiles, int top, int hidden, int inter,
+                                                                int act_kind) {
+  const int4 tile = tiles[blockIdx.x];  // (expert, first sorted row, rows, unused)
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int col = lane % 16, kg = lane / 16;
+  const int f0 = blockIdx.y * 64 + wave * 16;
+  if (tile.z <= 0 || f0 >= inter) return;
+  const int64_t w_row = (int64_t)tile.x * inter + min(f0 + col, inter - 1);
+  const bf16_t* gw = gate_w + w_row * hidden + 8 * kg;
+  const bf16_t* uw = up_w + w_row * hidden + 8 * kg;
+  const bf16_t* rows[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int r = mt * 16 + col;
+    rows[mt] = x + (int64_t)(order[tile.y + (r < tile.z ? r : 0)] / top) * ldx + 8 * kg;
+  }
+  f32x4 gs[MT], us[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) gs[mt] = us[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k = 0; k < hidden; k += 32) {
+    const bf16x8 g = *reinterpret_cast<const bf16x8*>(gw + k);
+    const bf16x8 u = *reinterpret_cast<const bf16x8*>(uw + k);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+      gs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g, a, gs[mt], 0, 0, 0);
+      us[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, a, us[mt], 0, 0, 0);
+    }
+  }
+  // a lane holds features f0 + 4 kg .. + 3 of the row mt * 16 + col
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int r = mt * 16 + col;
+    if (r >= tile.z) continue;
+    bf16_t* o = act + (int64_t)(tile.y + r) * inter + f0 + 4 * kg;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (f0 + 4 * kg + i < inter) o[i] = __float2bfloat16(act_of(gs[mt][i], act_kind) * us[mt][i]);
+  }
+}
+
+template <int MT>
+__global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__ y, const bf16_t* __restrict__ act,
+                                                             const bf16_t* __restrict__ down_w, const int* __restrict__ order,
+                                                             const float* __restrict__ weights, const int4* __restrict__ tiles,
+                                                             int top, int num_tokens, int hidden, int inter) {
+  const int4 tile = tiles[blockIdx.x];
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int col = lane % 16, kg = lane / 16;
+  const int n0 = blockIdx.y * 64 + wave * 16;
+  if (tile.z <= 0 || n0 >= hidden) return;
+  const bf16_t* w = down_w + ((int64_t)tile.x * hidden + min(n0 + col, hidden - 1)) * inter + 8 * kg;
+  const bf16_t* rows[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int r = mt * 16 + col;
+    rows[mt] = act + (int64_t)(tile.y + (r < tile.z ? r : 0)) * inter + 8 * kg;
+  }
+  f32x4 sums[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) sums[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k = 0; k < inter; k += 32) {
+    const bf16x8 wk = *reinterpret_cast<const bf16x8*>(w + k);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      sums[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wk, *reinterpret_cast<const bf16x8*>(rows[mt] + k), sums[mt], 0, 0, 0);
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int r = mt * 16 + col;
+    if (r >= tile.z) continue;
+    const int pair = order[tile.y + r];
+    const float weight = weights[pair];
+    float* o = y + ((int64_t)(pair % top) * num_tokens + pair / top) * hidden + n0 + 4 * kg;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n0 + 4 * kg + i < hidden) o[i] = weight * sums[mt][i];
+  }
+}
+
+// rows a tile holds for a step of that many pairs: 16 while an expert sees a few tokens, 64 in prompts
+extern "C" int pae_moe_tile_rows(int pairs) { return pairs <= 512 ? 16 : 64; }
+extern "C" int pae_moe_max_tiles(int pairs, int experts) {
+  const int rows = pae_moe_tile_rows(pairs);
+  return (pairs + rows - 1) / rows + experts;
+}
+extern "C" int pae_moe_tiles_supported(int hidden, int inter) { return hidden % 32 == 0 && inter % 32 == 0; }
+
+// `order` int32 [pairs], `tiles` int32 [pae_moe_max_tiles][4], `act` bfloat16 [pairs][inter] are work space;
+// y float32 [top][num_tokens][hidden] receives every pair's weighted output.
+extern "C" int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const void* gate_w, const void* up_w,
+                                     const void* down_w, const int* chosen, const float* weights, int num_tokens, int top,
+                                     int experts, int hidden, int inter, int act_kind, int* order, int* tiles, void* act,
+                                     hipStream_t stream) {
+  PAE_REQUIRE(top > 0 && experts > 0 && experts <= 4096, "experts: bad sizes top=%d experts=%d", top, experts);
+  PAE_REQUIRE(pae_moe_tiles_supported(hidden, inter), "experts: widths %d and %d are no multiples of 32", hidden, inter);
+  PAE_REQUIRE(ldx >= hidden && ldx % 8 == 0, "experts: row stride %lld", (long long)ldx);
+  if (num_tokens <= 0) return 0;
+  const int pairs = num_tokens * top;
+  const int tile_rows = pae_moe_tile_rows(pairs), max_tiles = pae_moe_max_tiles(pairs, experts);
+  moe_sort_kernel<<<1, 1024, (size_t)(4 * experts + 1) * sizeof(int), stream>>>(chosen, pairs, experts, tile_rows, order,
+                                                                               (int4*)tiles, max_tiles);
+  dim3 up_grid(max_tiles, (inter + 63) / 64), down_grid(max_tiles, (hidden + 63) / 64);
+  PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);
+  if (tile_rows == 16) {
+    moe_tiles_gate_up_kernel<1><<<up_grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
+                                                             (const bf16_t*)up_w, order, (const int4*)tiles, top, hidden, inter,
+                                                             act_kind);
+    moe_tiles_down_kernel<1><<<down_grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)down_w, order, weights,
+                                                            (const int4*)tiles, top, num_tokens, hidden, inter);
+  } else {
+    moe_tiles_gate_up_kernel<4><<<up_grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
+                                                             (const bf16_t*)up_w, order, (const int4*)tiles, top, hidden, inter,
+                                                             act_kind);
+    moe_tiles_down_kernel<4><<<down_grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)down_w, order, weights,
+                                                            (const int4*)tiles, top, num_tokens, hidden, inter);
+  }
+  return pae_check_launch("moe_experts_tiles");
 }

@@ -82,7 +82,7 @@ def _declare(lib) -> None:
         "pae_heads_product_few": [P, L, L, P, L, L, P, I, I, I, I, P],
         "pae_latent_attn_supported": [I, I, I],
         "pae_latent_attn_columns": [I, I],
-        "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P, P, P],
+        "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P, P, P, P],
         "pae_latent_attn_split": [],
         "pae_gated_act": [I, P, P, I, I, I, I, P],
         "pae_gemm_plain_batched": [I, I, P, L, L, P, L, L, P, L, P, I, I, I, I, I, P],
@@ -98,6 +98,10 @@ def _declare(lib) -> None:
         "pae_moe_route": [P, I, I, I, I, I, F, P, P, P],
         "pae_moe_gate_up": [I, P, P, L, P, P, P, I, I, I, I, I, P],
         "pae_moe_down": [I, P, P, P, P, P, I, I, I, I, P],
+        "pae_moe_tile_rows": [I],
+        "pae_moe_max_tiles": [I, I],
+        "pae_moe_tiles_supported": [I, I],
+        "pae_moe_experts_tiles": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
         "pae_sample_chunks": [I],
         "pae_sample_static": [P, P, L, P, P, I, I, P],
@@ -1143,14 +1147,16 @@ def latent_attn_tokens(num_heads: int, column_tiles: int) -> int:
 
 def latent_attn(out: torch.Tensor, q_full: torch.Tensor, latent: torch.Tensor, latent_t: torch.Tensor, tiles: torch.Tensor,
                 column_tiles: int, positions: torch.Tensor, block_tables: torch.Tensor, nh: int, rank: int, scale: float,
-                window: int = 0, chunked: bool = False) -> None:
+                window: int = 0, chunked: bool = False, sinks: Optional[torch.Tensor] = None) -> None:
     """Latent attention on the matrix cores.  `q_full` [T, nh * KD] holds per head the query folded into
     latent space and its rotated part; `latent` [block][bs][KD] and `latent_t` [block][rank][bs] are the
     cached rows and their transposed latents; tiles[i] = (table row, first flat token, tokens, 0) with at
     most `latent_attn_tokens(nh, column_tiles)` tokens; out[t, h * rank:(h + 1) * rank] receives the
-    weighted sums of the latents."""
+    weighted sums of the latents.  `sinks` float32 [nh]: exp(sink) joins each head's denominator."""
     _not_while_recording("latent_attn")
-    _gpu(out, q_full, latent, latent_t, tiles, positions, block_tables)
+    _gpu(out, q_full, latent, latent_t, tiles, positions, block_tables, sinks)
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
     T = q_full.shape[0]
     kd, bs = latent.shape[2], latent.shape[1]
     assert q_full.dtype == torch.bfloat16 == out.dtype == latent.dtype == latent_t.dtype
@@ -1170,7 +1176,8 @@ def latent_attn(out: torch.Tensor, q_full: torch.Tensor, latent: torch.Tensor, l
     _check(library().pae_latent_attn_bf16(
         out.data_ptr(), out.stride(0), q_full.data_ptr(), q_full.stride(0), latent.data_ptr(), latent_t.data_ptr(),
         tiles.data_ptr(), tiles.shape[0], column_tiles, positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
-        bs, nh, kd, rank, float(scale), int(window), 1 if chunked else 0, _ptr(part_acc), _ptr(part_ml), _stream()))
+        bs, nh, kd, rank, float(scale), int(window), 1 if chunked else 0, _ptr(part_acc), _ptr(part_ml), _ptr(sinks),
+        _stream()))
 
 
 def hyper_norm(streams: torch.Tensor, num_streams: int, y: Optional[torch.Tensor], layer_scale: Optional[torch.Tensor],
@@ -1503,8 +1510,9 @@ def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int, scale: flo
 
 def moe_experts(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor, chosen: torch.Tensor,
                 weights: torch.Tensor, activation: str = "silu") -> torch.Tensor:
-    """float32 [T, H]: for every token the weighted sum over its chosen experts of
-    W_down[e] (act(W_gate[e] x) * (W_up[e] x)); `gate_w`, `up_w` [E, F, H] and `down_w` [E, H, F] in x's type."""
+    """For every token the weighted sum over its chosen experts of W_down[e] (act(W_gate[e] x) * (W_up[e] x));
+    `gate_w`, `up_w` [E, F, H] and `down_w` [E, H, F] in x's type.  Returns float32 [T, H], or, from the
+    matrix-core kernels (bfloat16, widths in multiples of 32), float32 [top, T, H] whose `top` parts add up to it."""
     _not_while_recording("moe_experts")
     _gpu(x, gate_w, up_w, down_w, chosen, weights)
     T, H = x.shape
@@ -1517,8 +1525,17 @@ def moe_experts(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_
     assert weights.dtype == torch.float32 and weights.shape == chosen.shape and weights.is_contiguous()
     assert activation in ACTIVATIONS
     act = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
-    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
     lib = library()
+    if x.dtype == torch.bfloat16 and lib.pae_moe_tiles_supported(H, F) and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        parts = torch.empty((top, T, H), dtype=torch.float32, device=x.device)
+        order = torch.empty(T * top, dtype=torch.int32, device=x.device)
+        tiles = torch.empty((lib.pae_moe_max_tiles(T * top, E), 4), dtype=torch.int32, device=x.device)
+        _check(lib.pae_moe_experts_tiles(parts.data_ptr(), x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr(),
+                                         down_w.data_ptr(), chosen.data_ptr(), weights.data_ptr(), T, top, E, H, F,
+                                         ACTIVATIONS[activation], order.data_ptr(), tiles.data_ptr(), act.data_ptr(),
+                                         _stream()))
+        return parts
+    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
     _check(lib.pae_moe_gate_up(code_of(x.dtype), act.data_ptr(), x.data_ptr(), x.stride(0), gate_w.data_ptr(),
                                up_w.data_ptr(), chosen.data_ptr(), T, top, H, F, ACTIVATIONS[activation], _stream()))
     _check(lib.pae_moe_down(code_of(x.dtype), out.data_ptr(), act.data_ptr(), down_w.data_ptr(), chosen.data_ptr(),

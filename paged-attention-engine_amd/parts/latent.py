@@ -96,7 +96,7 @@ class LatentAttention(Part):
     @property
     def matrix_cores(self) -> bool:
         """Whether the attention runs on the matrix cores (then the pages also hold the latents transposed)."""
-        return not self.spec.sinks and K.latent_attn_supported(self.dtype, self.row_width, self.spec.kv_rank)
+        return K.latent_attn_supported(self.dtype, self.row_width, self.spec.kv_rank)
 
     def paged_spec(self):
         s = self.spec
@@ -164,7 +164,7 @@ class LatentAttention(Part):
             for name, column_tiles in (("single", 1), ("runs", 2)):
                 if tiles[name].numel():
                     K.latent_attn(summed, q_full, latent, latent_t, tiles[name], column_tiles, ctx.positions, table, H, C,
-                                  s.scale, s.window or 0, s.mask == "chunk")
+                                  s.scale, s.window or 0, s.mask == "chunk", self.sinks)
         else:
             K.paged_attention_masked(summed, q_full, latent, None, ctx.positions, ctx.tok_seq, table, H, 1, C + R, C, s.scale,
                                      s.window or 0, s.mask == "chunk", sinks=self.sinks)
