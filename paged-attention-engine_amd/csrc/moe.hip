@@ -220,7 +220,7 @@ extern "C" int pae_moe_down(int dtype, float* out, const void* act, const void* 
 // ---------------------------------------------------------------------------------------------------------------
 // The experts on the matrix cores (bfloat16, widths in multiples of 32).  The (token, expert) pairs of a step are
 // sorted by expert on the device, and every expert's pairs are cut into tiles of up to 16 MT rows; a workgroup takes one
-// tile and 64 output features, its four wavefronts 16 features each, so an expert's weights are streamed once per
+// tile and 64 or more output features, its four wavefronts a quarter each, so an expert's weights are streamed once per
 // tile: once in all for a step of a few tokens, and once per 16 MT of an expert's tokens in a prompt.  Which tile a
 // pair falls into changes nothing of its sums (k ascends in steps of 32 for every row by itself), so a token's
 // result does not depend on the batch.
@@ -266,7 +266,9 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
   for (int i = *total + threadIdx.x; i < max_tiles; i += 1024) tiles[i] = make_int4(0, 0, 0, 0);
 }
 
-template <int MT>
+// A wavefront holds MT tiles of 16 rows by NT tiles of 16 features: MT + NT (2 NT with gate and up) operand loads
+// feed MT NT (2 MT NT) matrix instructions in every step of 32 of k.
+template <int MT, int NT>
 __global__ __launch_bounds__(256) void moe_tiles_gate_up_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ x,
                                                                 int64_t ldx, const bf16_t* __restrict__ gate_w,
                                                                 const bf16_t* __restrict__ up_w, const int* __restrict__ order,
@@ -275,44 +277,62 @@ __global__ __launch_bounds__(256) void moe_tiles_gate_up_kernel(bf16_t* __restri
   const int4 tile = tiles[blockIdx.x];  // (expert, first sorted row, rows, unused)
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int col = lane % 16, kg = lane / 16;
-  const int f0 = blockIdx.y * 64 + wave * 16;
+  const int f0 = (blockIdx.y * 4 + wave) * 16 * NT;
   if (tile.z <= 0 || f0 >= inter) return;
-  const int64_t w_row = (int64_t)tile.x * inter + min(f0 + col, inter - 1);
-  const bf16_t* gw = gate_w + w_row * hidden + 8 * kg;
-  const bf16_t* uw = up_w + w_row * hidden + 8 * kg;
+  const bf16_t* gw[NT];
+  const bf16_t* uw[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int64_t w_row = (int64_t)tile.x * inter + min(f0 + 16 * nt + col, inter - 1);
+    gw[nt] = gate_w + w_row * hidden + 8 * kg;
+    uw[nt] = up_w + w_row * hidden + 8 * kg;
+  }
   const bf16_t* rows[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int r = mt * 16 + col;
     rows[mt] = x + (int64_t)(order[tile.y + (r < tile.z ? r : 0)] / top) * ldx + 8 * kg;
   }
-  f32x4 gs[MT], us[MT];
+  f32x4 gs[MT][NT], us[MT][NT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) gs[mt] = us[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) gs[mt][nt] = us[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 2
   for (int k = 0; k < hidden; k += 32) {
-    const bf16x8 g = *reinterpret_cast<const bf16x8*>(gw + k);
-    const bf16x8 u = *reinterpret_cast<const bf16x8*>(uw + k);
+    bf16x8 g[NT], u[NT], a[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 a = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
-      gs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g, a, gs[mt], 0, 0, 0);
-      us[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, a, us[mt], 0, 0, 0);
+    for (int nt = 0; nt < NT; ++nt) {
+      g[nt] = *reinterpret_cast<const bf16x8*>(gw[nt] + k);
+      u[nt] = *reinterpret_cast<const bf16x8*>(uw[nt] + k);
     }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a[mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        gs[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g[nt], a[mt], gs[mt][nt], 0, 0, 0);
+        us[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[nt], a[mt], us[mt][nt], 0, 0, 0);
+      }
   }
-  // a lane holds features f0 + 4 kg .. + 3 of the row mt * 16 + col
+  // a lane holds features f0 + 16 nt + 4 kg .. + 3 of the row mt * 16 + col
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int r = mt * 16 + col;
     if (r >= tile.z) continue;
-    bf16_t* o = act + (int64_t)(tile.y + r) * inter + f0 + 4 * kg;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (f0 + 4 * kg + i < inter) o[i] = __float2bfloat16(act_of(gs[mt][i], act_kind) * us[mt][i]);
+    for (int nt = 0; nt < NT; ++nt) {
+      const int f = f0 + 16 * nt + 4 * kg;
+      bf16_t* o = act + (int64_t)(tile.y + r) * inter + f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (f + i < inter) o[i] = __float2bfloat16(act_of(gs[mt][nt][i], act_kind) * us[mt][nt][i]);
+    }
   }
 }
 
-template <int MT>
+template <int MT, int NT>
 __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__ y, const bf16_t* __restrict__ act,
                                                              const bf16_t* __restrict__ down_w, const int* __restrict__ order,
                                                              const float* __restrict__ weights, const int4* __restrict__ tiles,
@@ -320,24 +340,34 @@ __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__
   const int4 tile = tiles[blockIdx.x];
   const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
   const int col = lane % 16, kg = lane / 16;
-  const int n0 = blockIdx.y * 64 + wave * 16;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * NT;
   if (tile.z <= 0 || n0 >= hidden) return;
-  const bf16_t* w = down_w + ((int64_t)tile.x * hidden + min(n0 + col, hidden - 1)) * inter + 8 * kg;
+  const bf16_t* w[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+    w[nt] = down_w + ((int64_t)tile.x * hidden + min(n0 + 16 * nt + col, hidden - 1)) * inter + 8 * kg;
   const bf16_t* rows[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int r = mt * 16 + col;
     rows[mt] = act + (int64_t)(tile.y + (r < tile.z ? r : 0)) * inter + 8 * kg;
   }
-  f32x4 sums[MT];
+  f32x4 sums[MT][NT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) sums[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) sums[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 2
   for (int k = 0; k < inter; k += 32) {
-    const bf16x8 wk = *reinterpret_cast<const bf16x8*>(w + k);
+    bf16x8 wk[NT], a[MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wk[nt] = *reinterpret_cast<const bf16x8*>(w[nt] + k);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) a[mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      sums[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wk, *reinterpret_cast<const bf16x8*>(rows[mt] + k), sums[mt], 0, 0, 0);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) sums[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wk[nt], a[mt], sums[mt][nt], 0, 0, 0);
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -345,10 +375,14 @@ __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__
     if (r >= tile.z) continue;
     const int pair = order[tile.y + r];
     const float weight = weights[pair];
-    float* o = y + ((int64_t)(pair % top) * num_tokens + pair / top) * hidden + n0 + 4 * kg;
+    float* row = y + ((int64_t)(pair % top) * num_tokens + pair / top) * hidden;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (n0 + 4 * kg + i < hidden) o[i] = weight * sums[mt][i];
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n = n0 + 16 * nt + 4 * kg;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < hidden) row[n + i] = weight * sums[mt][nt][i];
+    }
   }
 }
 
@@ -374,20 +408,19 @@ extern "C" int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const
   const int tile_rows = pae_moe_tile_rows(pairs), max_tiles = pae_moe_max_tiles(pairs, experts);
   moe_sort_kernel<<<1, 1024, (size_t)(4 * experts + 1) * sizeof(int), stream>>>(chosen, pairs, experts, tile_rows, order,
                                                                                (int4*)tiles, max_tiles);
-  dim3 up_grid(max_tiles, (inter + 63) / 64), down_grid(max_tiles, (hidden + 63) / 64);
-  PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);
-  if (tile_rows == 16) {
-    moe_tiles_gate_up_kernel<1><<<up_grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
-                                                             (const bf16_t*)up_w, order, (const int4*)tiles, top, hidden, inter,
-                                                             act_kind);
-    moe_tiles_down_kernel<1><<<down_grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)down_w, order, weights,
-                                                            (const int4*)tiles, top, num_tokens, hidden, inter);
-  } else {
-    moe_tiles_gate_up_kernel<4><<<up_grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
-                                                             (const bf16_t*)up_w, order, (const int4*)tiles, top, hidden, inter,
-                                                             act_kind);
-    moe_tiles_down_kernel<4><<<down_grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)down_w, order, weights,
-                                                            (const int4*)tiles, top, num_tokens, hidden, inter);
-  }
+#define MOE_TILES(MT, UP_NT, DOWN_NT)                                                                                      \
+  do {                                                                                                                     \
+    dim3 up_grid(max_tiles, (inter + 64 * UP_NT - 1) / (64 * UP_NT)), down_grid(max_tiles, (hidden + 64 * DOWN_NT - 1) / (64 * DOWN_NT)); \
+    PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);      \
+    moe_tiles_gate_up_kernel<MT, UP_NT><<<up_grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)x, ldx,                   \
+                                                                      (const bf16_t*)gate_w, (const bf16_t*)up_w, order,    \
+                                                                      (const int4*)tiles, top, hidden, inter, act_kind);    \
+    moe_tiles_down_kernel<MT, DOWN_NT><<<down_grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)down_w, order,  \
+                                                                       weights, (const int4*)tiles, top, num_tokens, hidden, \
+                                                                       inter);                                              \
+  } while (0)
+  if (tile_rows == 16) MOE_TILES(1, 1, 1);
+  else MOE_TILES(4, 2, 4);
+#undef MOE_TILES
   return pae_check_launch("moe_experts_tiles");
 }
