@@ -31,18 +31,51 @@ __global__ __launch_bounds__(256) void project_f32_kernel(float* __restrict__ ou
   if (lane == 0) out[t * ldo + n] = sum + (bias ? load_param(bias, b_is_f32, n) : 0.f);
 }
 
+// The same sums with 16-byte loads, for rows and widths that allow them: a workgroup takes one row, its four
+// wavefronts the outputs in turn; a lane adds its 8 (or 4) consecutive k of every 64-lane stretch, then the lanes meet.
+template <typename T>
+__global__ __launch_bounds__(256) void project_f32_wide_kernel(float* __restrict__ out, int64_t ldo, const T* __restrict__ A,
+                                                               int64_t lda, const T* __restrict__ W,
+                                                               const void* __restrict__ bias, int b_is_f32, int N, int K) {
+  constexpr int VEC = 16 / sizeof(T);
+  struct alignas(16) Chunk { T v[VEC]; };
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
+  const T* a = A + t * lda;
+  for (int n = wave; n < N; n += 4) {
+    const T* w = W + (int64_t)n * K;
+    float sum = 0.f;
+    for (int k = lane * VEC; k < K; k += PAE_WAVE * VEC) {
+      const Chunk x = *reinterpret_cast<const Chunk*>(a + k);
+      const Chunk y = *reinterpret_cast<const Chunk*>(w + k);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) sum = fmaf(to_f32(x.v[i]), to_f32(y.v[i]), sum);
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) out[t * ldo + n] = sum + (bias ? load_param(bias, b_is_f32, n) : 0.f);
+  }
+}
+
 extern "C" int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A, int64_t lda, const void* W,
                                const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream) {
   PAE_REQUIRE(N > 0 && K > 0 && N <= 4 * 65535, "float32 projection: bad sizes N=%d K=%d", N, K);
   PAE_REQUIRE(ldo >= N && lda >= K, "float32 projection: row strides too small");
+  PAE_REQUIRE(dtype == PAE_F32 || dtype == PAE_BF16, "float32 projection: unknown dtype code %d", dtype);
   if (M <= 0) return 0;
+  const int vec = dtype == PAE_F32 ? 4 : 8;
+  const bool wide = K % vec == 0 && lda % vec == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0;
   dim3 grid(M, (N + 3) / 4);
-  if (dtype == PAE_F32)
-    project_f32_kernel<float><<<grid, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K);
-  else if (dtype == PAE_BF16)
-    project_f32_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K);
-  else
-    return pae_fail("float32 projection: unknown dtype code %d", dtype);
+  if (dtype == PAE_F32) {
+    if (wide)
+      project_f32_wide_kernel<float><<<M, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K);
+    else
+      project_f32_kernel<float><<<grid, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K);
+  } else {
+    if (wide)
+      project_f32_wide_kernel<bf16_t><<<M, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K);
+    else
+      project_f32_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K);
+  }
   return pae_check_launch("project_f32");
 }
 
@@ -298,23 +331,41 @@ __global__ __launch_bounds__(256) void moe_tiles_gate_up_kernel(bf16_t* __restri
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) gs[mt][nt] = us[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-  for (int k = 0; k < hidden; k += 32) {
-    bf16x8 g[NT], u[NT], a[MT];
+  // operands of the step after are on their way while a step's matrix instructions run; the loop's loads are
+  // unconditional and the last step stands by itself
+  bf16x8 g[2][NT], u[2][NT], a[2][MT];
+  auto load = [&](int set, int k) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      g[nt] = *reinterpret_cast<const bf16x8*>(gw[nt] + k);
-      u[nt] = *reinterpret_cast<const bf16x8*>(uw[nt] + k);
+      g[set][nt] = *reinterpret_cast<const bf16x8*>(gw[nt] + k);
+      u[set][nt] = *reinterpret_cast<const bf16x8*>(uw[nt] + k);
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) a[mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+    for (int mt = 0; mt < MT; ++mt) a[set][mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+  };
+  auto multiply = [&](int set) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        gs[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g[nt], a[mt], gs[mt][nt], 0, 0, 0);
-        us[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[nt], a[mt], us[mt][nt], 0, 0, 0);
+        gs[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g[set][nt], a[set][mt], gs[mt][nt], 0, 0, 0);
+        us[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[set][nt], a[set][mt], us[mt][nt], 0, 0, 0);
       }
+  };
+  load(0, 0);
+  int k = 0;
+  for (; k + 64 < hidden; k += 64) {
+    load(1, k + 32);
+    multiply(0);
+    load(0, k + 64);
+    multiply(1);
+  }
+  if (k + 32 < hidden) {
+    load(1, k + 32);
+    multiply(0);
+    multiply(1);
+  } else {
+    multiply(0);
   }
   // a lane holds features f0 + 16 nt + 4 kg .. + 3 of the row mt * 16 + col
 #pragma unroll
@@ -357,17 +408,34 @@ __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) sums[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-  for (int k = 0; k < inter; k += 32) {
-    bf16x8 wk[NT], a[MT];
+  bf16x8 wk[2][NT], a[2][MT];
+  auto load = [&](int set, int k) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) wk[nt] = *reinterpret_cast<const bf16x8*>(w[nt] + k);
+    for (int nt = 0; nt < NT; ++nt) wk[set][nt] = *reinterpret_cast<const bf16x8*>(w[nt] + k);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) a[mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+    for (int mt = 0; mt < MT; ++mt) a[set][mt] = *reinterpret_cast<const bf16x8*>(rows[mt] + k);
+  };
+  auto multiply = [&](int set) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) sums[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wk[nt], a[mt], sums[mt][nt], 0, 0, 0);
+      for (int nt = 0; nt < NT; ++nt)
+        sums[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wk[set][nt], a[set][mt], sums[mt][nt], 0, 0, 0);
+  };
+  load(0, 0);
+  int k = 0;
+  for (; k + 64 < inter; k += 64) {
+    load(1, k + 32);
+    multiply(0);
+    load(0, k + 64);
+    multiply(1);
+  }
+  if (k + 32 < inter) {
+    load(1, k + 32);
+    multiply(0);
+    multiply(1);
+  } else {
+    multiply(0);
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
