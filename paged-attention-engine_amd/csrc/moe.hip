@@ -31,18 +31,21 @@ __global__ __launch_bounds__(256) void project_f32_kernel(float* __restrict__ ou
   if (lane == 0) out[t * ldo + n] = sum + (bias ? load_param(bias, b_is_f32, n) : 0.f);
 }
 
-// The same sums with 16-byte loads, for rows and widths that allow them: a workgroup takes one row, its four
-// wavefronts the outputs in turn; a lane adds its 8 (or 4) consecutive k of every 64-lane stretch, then the lanes meet.
+// The same sums with 16-byte loads, for rows and widths that allow them: a workgroup takes one row and `per_wave`
+// outputs for each of its four wavefronts (all of a row's outputs in steps of many rows, one each in steps of
+// few); a lane adds its 8 (or 4) consecutive k of every 64-lane stretch, then the lanes meet.
 template <typename T>
 __global__ __launch_bounds__(256) void project_f32_wide_kernel(float* __restrict__ out, int64_t ldo, const T* __restrict__ A,
                                                                int64_t lda, const T* __restrict__ W,
-                                                               const void* __restrict__ bias, int b_is_f32, int N, int K) {
+                                                               const void* __restrict__ bias, int b_is_f32, int N, int K,
+                                                               int per_wave) {
   constexpr int VEC = 16 / sizeof(T);
   struct alignas(16) Chunk { T v[VEC]; };
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
   const T* a = A + t * lda;
-  for (int n = wave; n < N; n += 4) {
+  const int first = blockIdx.y * 4 * per_wave + wave;
+  for (int n = first; n < N && n < first + 4 * per_wave; n += 4) {
     const T* w = W + (int64_t)n * K;
     float sum = 0.f;
     for (int k = lane * VEC; k < K; k += PAE_WAVE * VEC) {
@@ -65,14 +68,16 @@ extern "C" int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A
   const int vec = dtype == PAE_F32 ? 4 : 8;
   const bool wide = K % vec == 0 && lda % vec == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0;
   dim3 grid(M, (N + 3) / 4);
+  const int per_wave = M >= 512 ? (N + 3) / 4 : 1;
+  dim3 wide_grid(M, (N + 4 * per_wave - 1) / (4 * per_wave));
   if (dtype == PAE_F32) {
     if (wide)
-      project_f32_wide_kernel<float><<<M, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K);
+      project_f32_wide_kernel<float><<<wide_grid, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K, per_wave);
     else
       project_f32_kernel<float><<<grid, 256, 0, stream>>>(out, ldo, (const float*)A, lda, (const float*)W, bias, b_is_f32, N, K);
   } else {
     if (wide)
-      project_f32_wide_kernel<bf16_t><<<M, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K);
+      project_f32_wide_kernel<bf16_t><<<wide_grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K, per_wave);
     else
       project_f32_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)A, lda, (const bf16_t*)W, bias, b_is_f32, N, K);
   }
@@ -454,10 +459,137 @@ __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__
   }
 }
 
-// rows a tile holds for a step of that many pairs: 16 while an expert sees a few tokens, 64 in prompts
-extern "C" int pae_moe_tile_rows(int pairs) { return pairs <= 512 ? 16 : 64; }
+// The same two products for prompts, where an expert sees hundreds of tokens: a workgroup takes a tile of 128 rows
+// and 128 features with gate and up (or 256 output features of the down product), and its operands pass through LDS:
+// every 64 of k, the 256 threads fetch 128 rows of activations and 256 rows of weights, a whole 128-byte line a row, into
+// registers while the step before is multiplied, and then write them to LDS (rows 144 bytes apart, so that the 16-byte
+// reads of a wavefront's lanes fall on all banks).  The four wavefronts are two by two: 64 rows by 64 features with gate
+// and up (or 128 features), 64 matrix instructions for 24 reads of LDS a step.  Two barriers a step.
+#define MOE_BIG_ROWS 128
+#define MOE_BIG_K 64
+#define MOE_LDS_STRIDE 72  // bf16 from a row of 64 to the next in LDS
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_big_tiles_kernel(bf16_t* __restrict__ act_out, float* __restrict__ y,
+                                                            const bf16_t* __restrict__ a_rows, int64_t lda,
+                                                            const bf16_t* __restrict__ w_first, const bf16_t* __restrict__ w_second,
+                                                            const int* __restrict__ order, const float* __restrict__ weights,
+                                                            const int4* __restrict__ tiles, int top, int num_tokens, int K,
+                                                            int N, int act_kind) {
+  // GATED: a_rows = x (row of a pair = its token), w_first / w_second = gate / up [E][N][K], N = the experts' width;
+  // else: a_rows = act in sorted order, w_first = down [E][N][K], N = the hidden width
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[MOE_BIG_ROWS * MOE_LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_w[256 * MOE_LDS_STRIDE];
+  const int4 tile = tiles[blockIdx.x];  // (expert, first sorted row, rows, unused)
+  if (tile.z <= 0) return;
+  constexpr int FEATURES = GATED ? 128 : 256;  // output features a workgroup takes
+  const int n_base = blockIdx.y * FEATURES;
+  const int tid = threadIdx.x, lane = tid % PAE_WAVE, wave = tid / PAE_WAVE;
+  const int col = lane % 16, kg = lane / 16;
+  const int wr = wave / 2, wc = wave % 2;
+  // what this thread fetches: 16 bytes (piece tid % 8) of rows tid / 8 + 32 j
+  const int piece = tid % 8, frow = tid / 8;
+  const bf16_t* a_src[4];
+  const bf16_t* w_src[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = frow + 32 * j;
+    const int sorted = tile.y + (r < tile.z ? r : 0);
+    const int64_t row = GATED ? order[sorted] / top : sorted;
+    a_src[j] = a_rows + row * lda + 8 * piece;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int r = frow + 32 * j;  // row of the 256 in LDS: gated, the first 128 are gate's features, the rest up's
+    const int n = min(n_base + (GATED ? r % 128 : r), N - 1);
+    const bf16_t* w = (GATED && r >= 128) ? w_second : w_first;
+    w_src[j] = w + ((int64_t)tile.x * N + n) * K + 8 * piece;
+  }
+  f32x4 acc[4][8];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 fa[4], fw[8];
+  auto fetch = [&](int k) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fa[j] = *reinterpret_cast<const bf16x8*>(a_src[j] + k);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(w_src[j] + k);
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(&lds_a[(frow + 32 * j) * MOE_LDS_STRIDE + 8 * piece]) = fa[j];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) *reinterpret_cast<bf16x8*>(&lds_w[(frow + 32 * j) * MOE_LDS_STRIDE + 8 * piece]) = fw[j];
+  };
+  auto multiply = [&]() {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      bf16x8 a[4], w[8];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        a[mt] = *reinterpret_cast<const bf16x8*>(&lds_a[(wr * 64 + 16 * mt + col) * MOE_LDS_STRIDE + 32 * half + 8 * kg]);
+#pragma unroll
+      for (int nt = 0; nt < 8; ++nt) {
+        // gated: tiles 0..3 are gate's features wc * 64 + 16 nt, tiles 4..7 the same features of up
+        const int row = GATED ? (nt / 4) * 128 + wc * 64 + 16 * (nt % 4) + col : wc * 128 + 16 * nt + col;
+        w[nt] = *reinterpret_cast<const bf16x8*>(&lds_w[row * MOE_LDS_STRIDE + 32 * half + 8 * kg]);
+      }
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[nt], a[mt], acc[mt][nt], 0, 0, 0);
+    }
+  };
+  fetch(0);
+  stage();
+  __syncthreads();
+  const int steps = K / MOE_BIG_K;
+  for (int s = 1; s < steps; ++s) {
+    fetch(MOE_BIG_K * s);  // on its way while the step before is multiplied
+    multiply();
+    __syncthreads();       // everyone has read the step before
+    stage();
+    __syncthreads();
+  }
+  multiply();
+  // a lane holds features 16 nt + 4 kg .. + 3 (of its wavefront's) of the row wr * 64 + 16 mt + col
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int r = wr * 64 + 16 * mt + col;
+    if (r >= tile.z) continue;
+    if (GATED) {
+      bf16_t* o = act_out + (int64_t)(tile.y + r) * N;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int f = n_base + wc * 64 + 16 * nt + 4 * kg;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (f + i < N) o[f + i] = __float2bfloat16(act_of(acc[mt][nt][i], act_kind) * acc[mt][nt + 4][i]);
+      }
+    } else {
+      const int pair = order[tile.y + r];
+      const float weight = weights[pair];
+      float* o = y + ((int64_t)(pair % top) * num_tokens + pair / top) * N;
+#pragma unroll
+      for (int nt = 0; nt < 8; ++nt) {
+        const int n = n_base + wc * 128 + 16 * nt + 4 * kg;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) o[n + i] = weight * acc[mt][nt][i];
+      }
+    }
+  }
+}
+
+// rows a tile holds for a step of that many pairs: 16 while an expert sees a few tokens, 64 in portions, 128 in prompts
+static int moe_tile_rows(int pairs, int hidden, int inter) {
+  if (pairs <= 512) return 16;
+  return (pairs > 4096 && hidden % MOE_BIG_K == 0 && inter % MOE_BIG_K == 0) ? MOE_BIG_ROWS : 64;
+}
+extern "C" int pae_moe_tile_rows(int pairs) { return pairs <= 512 ? 16 : (pairs <= 4096 ? 64 : MOE_BIG_ROWS); }
 extern "C" int pae_moe_max_tiles(int pairs, int experts) {
-  const int rows = pae_moe_tile_rows(pairs);
+  const int rows = pairs <= 512 ? 16 : 64;  // the smallest tiles such a step may get: the most tiles there can be
   return (pairs + rows - 1) / rows + experts;
 }
 extern "C" int pae_moe_tiles_supported(int hidden, int inter) { return hidden % 32 == 0 && inter % 32 == 0; }
@@ -473,7 +605,7 @@ extern "C" int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const
   PAE_REQUIRE(ldx >= hidden && ldx % 8 == 0, "experts: row stride %lld", (long long)ldx);
   if (num_tokens <= 0) return 0;
   const int pairs = num_tokens * top;
-  const int tile_rows = pae_moe_tile_rows(pairs), max_tiles = pae_moe_max_tiles(pairs, experts);
+  const int tile_rows = moe_tile_rows(pairs, hidden, inter), max_tiles = pae_moe_max_tiles(pairs, experts);
   moe_sort_kernel<<<1, 1024, (size_t)(4 * experts + 1) * sizeof(int), stream>>>(chosen, pairs, experts, tile_rows, order,
                                                                                (int4*)tiles, max_tiles);
 #define MOE_TILES(MT, UP_NT, DOWN_NT)                                                                                      \
@@ -488,7 +620,17 @@ extern "C" int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const
                                                                        inter);                                              \
   } while (0)
   if (tile_rows == 16) MOE_TILES(1, 1, 1);
-  else MOE_TILES(4, 2, 4);
+  else if (tile_rows == 64) MOE_TILES(4, 2, 4);
+  else {
+    dim3 up_grid(max_tiles, (inter + 127) / 128), down_grid(max_tiles, (hidden + 255) / 256);
+    PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);
+    moe_big_tiles_kernel<true><<<up_grid, 256, 0, stream>>>((bf16_t*)act, nullptr, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
+                                                            (const bf16_t*)up_w, order, weights, (const int4*)tiles, top,
+                                                            num_tokens, hidden, inter, act_kind);
+    moe_big_tiles_kernel<false><<<down_grid, 256, 0, stream>>>(nullptr, y, (const bf16_t*)act, inter, (const bf16_t*)down_w,
+                                                               nullptr, order, weights, (const int4*)tiles, top, num_tokens,
+                                                               inter, hidden, act_kind);
+  }
 #undef MOE_TILES
   return pae_check_launch("moe_experts_tiles");
 }

@@ -35,7 +35,11 @@ __global__ __launch_bounds__(256) void sum_norm2_kernel(float* __restrict__ resi
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += 256) {
     float v = x[i];
-    for (int j = 0; j < terms.count; ++j) {
+    // (the terms are walked with constant indices: an index that is only known at run time would move the
+    // whole description from the kernel's arguments into private memory)
+#pragma unroll
+    for (int j = 0; j < PAE_MAX_TERMS; ++j) {
+      if (j >= terms.count) break;
       float sum = 0.f;
       if (terms.is_f32[j]) {
         const float* p = (const float*)terms.ptr[j] + src * hidden + i;

@@ -390,10 +390,12 @@ def test_routing_passes_over_a_better_expert_of_a_dropped_group():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [dict(T=5, E=6, top=2, H=64, F=32), dict(T=70, E=4, top=1, H=96, F=64), dict(T=700, E=7, top=3, H=64, F=96),
-                                  dict(T=9, E=5, top=2, H=40, F=24)])
+                                  dict(T=9, E=5, top=2, H=40, F=24), dict(T=1500, E=6, top=3, H=96, F=160),
+                                  dict(T=2100, E=3, top=2, H=288, F=64)])
 def test_experts_by_pairs_and_by_sorted_tiles(dtype, case):
-    """Few tokens (tiles of 16 rows), hundreds (tiles of 64, experts with many tiles and one with no token at all), and
-    widths the matrix-core kernels do not take."""
+    """Few tokens (tiles of 16 rows), hundreds (tiles of 64), thousands (tiles of 128 staged through LDS, widths that
+    end inside a workgroup's features), experts with many tiles and one with no token at all, and widths the matrix-core
+    kernels do not take."""
     T, E, top, H, F = (case[k] for k in ("T", "E", "top", "H", "F"))
     gen = torch.Generator().manual_seed(T)
     x = (torch.randn((T, H), generator=gen)).to(dtype)
