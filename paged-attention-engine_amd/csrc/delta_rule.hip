@@ -93,13 +93,15 @@ __global__ __launch_bounds__(128) void delta_prepare_kernel(
     const T* b_row = b_in + (int64_t)t * b_stride;
     const T* a_row = a_in + (int64_t)t * a_stride;
     for (int h = threadIdx.x; h < H; h += 128) beta_out[(int64_t)t * H + h] = 1.0f / (1.0f + expf(-to_f32(b_row[h])));
-    if (channel_decay) {  // one decay per head and key channel, [H][D]
-      for (int c = threadIdx.x; c < H * D; c += 128)
-        decay_out[(int64_t)t * H * D + c] = expf(-expf(a_log[c / D]) * softplus_f(to_f32(a_row[c]) + dt_bias[c]));
-    } else {
+    if (!channel_decay) {
       for (int h = threadIdx.x; h < H; h += 128)
         decay_out[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(to_f32(a_row[h]) + dt_bias[h]));
     }
+  }
+  if (channel_decay) {  // one decay per head and key channel, [H][D]: every segment's workgroup takes its share
+    const T* a_row = a_in + (int64_t)t * a_stride;
+    for (int c = seg * 128 + threadIdx.x; c < H * D; c += gridDim.y * 128)
+      decay_out[(int64_t)t * H * D + c] = expf(-expf(a_log[c / D]) * softplus_f(to_f32(a_row[c]) + dt_bias[c]));
   }
 }
 
