@@ -23,6 +23,23 @@ struct SumTerms {
 };
 
 template <typename T>
+__device__ __forceinline__ void load4(const T* p, float (&v)[4]);
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float (&v)[4]) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+template <>
+__device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float (&v)[4]) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);  // a bfloat16 is the upper half of a float
+  v[0] = __uint_as_float(raw.x << 16); v[1] = __uint_as_float(raw.x & 0xffff0000u);
+  v[2] = __uint_as_float(raw.y << 16); v[3] = __uint_as_float(raw.y & 0xffff0000u);
+}
+
+// VEC: four consecutive features a thread and trip (widths in multiples of four), else one.  The first pass only
+// reads memory (the new row goes to LDS), so that nothing keeps its loads from being in flight together; the
+// second writes the stream and the norms.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void sum_norm2_kernel(float* __restrict__ residual, SumTerms terms,
                                                         const void* __restrict__ w1, int w1_is_f32,
                                                         const void* __restrict__ w2, int w2_is_f32, float eps,
@@ -30,34 +47,50 @@ __global__ __launch_bounds__(256) void sum_norm2_kernel(float* __restrict__ resi
                                                         T* __restrict__ out2, int hidden, int write_residual) {
   extern __shared__ float row_lds[];  // [hidden]
   __shared__ float scratch[4];
+  constexpr int W = VEC ? 4 : 1;
   const int64_t src = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = residual + src * hidden;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    float v = x[i];
+  for (int i = threadIdx.x * W; i < hidden; i += 256 * W) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (VEC) load4<float>(x + i, v);
+    else v[0] = x[i];
     // (the terms are walked with constant indices: an index that is only known at run time would move the
     // whole description from the kernel's arguments into private memory)
 #pragma unroll
     for (int j = 0; j < PAE_MAX_TERMS; ++j) {
       if (j >= terms.count) break;
-      float sum = 0.f;
+      float sum[4] = {0.f, 0.f, 0.f, 0.f};
       if (terms.is_f32[j]) {
         const float* p = (const float*)terms.ptr[j] + src * hidden + i;
-        for (int part = 0; part < terms.parts[j]; ++part) sum += p[part * terms.part_stride[j]];
+        for (int part = 0; part < terms.parts[j]; ++part) {
+          float t[4] = {0.f, 0.f, 0.f, 0.f};
+          if (VEC) load4<float>(p + part * terms.part_stride[j], t);
+          else t[0] = p[part * terms.part_stride[j]];
+#pragma unroll
+          for (int e = 0; e < W; ++e) sum[e] += t[e];
+        }
       } else {
-        sum = to_f32(((const T*)terms.ptr[j])[src * hidden + i]);
+        const T* p = (const T*)terms.ptr[j] + src * hidden + i;
+        if (VEC) load4<T>(p, sum);
+        else sum[0] = to_f32(p[0]);
       }
-      v += terms.scale[j] * sum;
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] += terms.scale[j] * sum[e];
     }
-    if (write_residual) x[i] = v;
-    row_lds[i] = v;
-    ss = fmaf(v, v, ss);
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+      row_lds[i + e] = v[e];
+      ss = fmaf(v[e], v[e], ss);
+    }
   }
   ss = block_sum<4>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
   const int64_t dst = (int64_t)blockIdx.x * hidden;
   for (int i = threadIdx.x; i < hidden; i += 256) {
-    const float n = row_lds[i] * inv;
+    const float v = row_lds[i];
+    if (write_residual) x[i] = v;
+    const float n = v * inv;
     if (out1) out1[dst + i] = from_f32<T>(n * load_param(w1, w1_is_f32, i));
     if (out2) out2[dst + i] = from_f32<T>(n * load_param(w2, w2_is_f32, i));
   }
@@ -83,11 +116,18 @@ extern "C" int pae_sum_norm2(int dtype, float* residual, int num_terms, const vo
     terms.scale[j] = term_scale[j];
   }
   const size_t lds = (size_t)hidden * sizeof(float);
-  if (dtype == PAE_F32)
-    sum_norm2_kernel<float><<<num_rows, 256, lds, stream>>>(residual, terms, w1, w1_is_f32, w2, w2_is_f32, eps, rows,
-                                                            (float*)out1, (float*)out2, hidden, rows ? 0 : write_residual);
-  else
-    sum_norm2_kernel<bf16_t><<<num_rows, 256, lds, stream>>>(residual, terms, w1, w1_is_f32, w2, w2_is_f32, eps, rows,
-                                                             (bf16_t*)out1, (bf16_t*)out2, hidden, rows ? 0 : write_residual);
+  bool vec = hidden % 4 == 0 && (uintptr_t)residual % 16 == 0;
+  for (int j = 0; j < num_terms; ++j) vec = vec && (uintptr_t)term_ptr[j] % 16 == 0 && term_part_stride[j] % 4 == 0;
+#define SUM_NORM2(T, VEC)                                                                                          \
+  sum_norm2_kernel<T, VEC><<<num_rows, 256, lds, stream>>>(residual, terms, w1, w1_is_f32, w2, w2_is_f32, eps, rows, \
+                                                           (T*)out1, (T*)out2, hidden, rows ? 0 : write_residual)
+  if (dtype == PAE_F32) {
+    if (vec) SUM_NORM2(float, true);
+    else SUM_NORM2(float, false);
+  } else {
+    if (vec) SUM_NORM2(bf16_t, true);
+    else SUM_NORM2(bf16_t, false);
+  }
+#undef SUM_NORM2
   return pae_check_launch("sum_norm2");
 }
