@@ -116,8 +116,13 @@ class GatedDeltaMixer(Part):
     def bind(self, prefix, weights):
         s = self.spec
         _, two = s.low_rank_suffixes
-        self.proj = Linear(self.matrix(torch.cat([weights[prefix + name + s.weight_suffix]
-                                                  for name, _ in self._projections()], dim=0)))
+        stacked = [weights[prefix + name + s.weight_suffix] for name, _ in self._projections()]
+        rows = sum(w.shape[0] for w in stacked)
+        if rows % 8:
+            # rows of zeros behind the last projection: the product's rows then start on 16-byte boundaries, which
+            # the few-row kernels want of the views that the narrow products read
+            stacked.append(torch.zeros((8 - rows % 8, s.hidden_size), dtype=stacked[0].dtype, device=stacked[0].device))
+        self.proj = Linear(self.matrix(torch.cat(stacked, dim=0)))
         self.gate_up = self.decay_up = None
         if s.gate_rank is not None:
             self.gate_up = Linear(self.matrix(weights[prefix + s.gate_name + two + s.weight_suffix]))
