@@ -10,8 +10,9 @@ scheduler, and through `bin/trace_run` as a program.
 Routing is a choice between numbers: where two experts' scores are within a rounding of each other,
 reduced precision may choose the other one, and everything after differs.  In float32 the engine must
 choose as the plain implementation does.  In bfloat16 the engine's choices are read out (a tap on the
-feed-forward), must equal the plain ones wherever the plain margin is clear, and the plain logits the
-engine is compared with are those of its own choices.
+feed-forward); the plain implementation is run on those choices, which gives the logits the engine is
+compared with and, layer by layer, what the plain implementation would have chosen itself on the same
+stream: wherever its margin is clear, the engine's choice must be that one.
 """
 
 import json
@@ -139,38 +140,26 @@ class Replay:
         if self.dtype == "float32":
             return check(got, want, "float32", what)
         cfg, weights = weights_of(self.folders, self.name)
-        own = plain.forward(weights, cfg, tokens, torch.float64, routing=routing)
-        choices = _plain_choices(self.folders, self.name, tokens)
-        for layer, margin in zip(moe_layers(cfg), margins):
-            clear = margin >= CLEAR_MARGIN
-            assert torch.equal(routing[layer][clear].sort(-1).values, choices[layer][clear].sort(-1).values), \
-                f"{what}: layer {layer} routes a token with a clear margin otherwise than the plain implementation"
-        return check(got, own, "bfloat16", what, rounding_alone(self.folders, self.name, tokens, own, routing))
-
-
-_CHOICES = {}
-
-
-def _plain_choices(folders, name, tokens):
-    """{layer: experts [T, top]} the plain implementation chooses on these tokens."""
-    key = (name, tuple(tokens))
-    if key not in _CHOICES:
-        cfg, weights = weights_of(folders, name)
-        taken = {}
+        # the plain implementation on the engine's choices; on the way, what it would have chosen itself at every
+        # layer (given the engine's choices in the layers before) and by what margin
+        free, own_margins = [], []
         original = plain.route
 
         def spy(z, router, margins=None):
             chosen, w = original(z, router, margins)
-            taken[len(taken)] = chosen
+            free.append(chosen)
             return chosen, w
 
         plain.route = spy
         try:
-            plain.forward(weights, cfg, tokens, torch.float64)
+            own = plain.forward(weights, cfg, tokens, torch.float64, margins=own_margins, routing=routing)
         finally:
             plain.route = original
-        _CHOICES[key] = {layer: taken[j] for j, layer in enumerate(moe_layers(cfg))}
-    return _CHOICES[key]
+        for layer, chosen, margin in zip(moe_layers(cfg), free, own_margins):
+            clear = margin >= CLEAR_MARGIN
+            assert torch.equal(routing[layer][clear].sort(-1).values, chosen[clear].sort(-1).values), \
+                f"{what}: layer {layer} routes a token with a clear margin otherwise than the plain implementation"
+        return check(got, own, "bfloat16", what, rounding_alone(self.folders, self.name, tokens, own, routing))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
