@@ -369,3 +369,26 @@ def test_the_program_replays_a_trace(folders, tmp_path):
     last = np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1)
     check(first, want[[0, 19]], "float32", "trace_run step 0")
     check(last, want[[36]], "float32", "trace_run step 2")
+
+
+def test_the_command_line_generates_and_samples(folders, tmp_path):
+    """`python -m paged_attention_engine_amd` on a model folder: greedy tokens of two prompts are the plain ones; with a
+    temperature the same seed gives the same tokens twice and another seed gives others."""
+    cfg, weights = weights_of(folders, "W")
+    prompts = [M.tokens_for("W", 19, salt=5), M.tokens_for("W", 7, salt=6)]
+    want = [plain.greedy_generate(weights, cfg, p, 6, torch.float64)[0] for p in prompts]
+
+    def run(*extra):
+        cmd = [sys.executable, "-m", "paged_attention_engine_amd", "--model", folders["W"], "--dtype", "float32", "--max-new-tokens", "6",
+               "--num-blocks", "16", "--max-num-seqs", "2"]
+        for p in prompts:
+            cmd += ["--prompt-ids", ",".join(map(str, p))]
+        proc = subprocess.run(cmd + list(extra), capture_output=True, text=True, timeout=600, cwd=ROOT)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        lines = [json.loads(line) for line in proc.stdout.splitlines() if line.startswith("{")]
+        return [line["token_ids"] for line in lines]
+
+    assert run() == want
+    first = run("--temperature", "0.9", "--sample-seed", "3")
+    assert first == run("--temperature", "0.9", "--sample-seed", "3")
+    assert first != run("--temperature", "0.9", "--sample-seed", "4") and first != want
