@@ -265,9 +265,11 @@ extern "C" int pae_moe_down(int dtype, float* out, const void* act, const void* 
 //
 //   moe_sort            counts, offsets and tiles by expert (one workgroup; the order of an expert's pairs among
 //                       themselves is whatever the counters' turn gives, and does not matter)
-//   moe_tiles_gate_up   act(W_gate x) * (W_up x) for a tile's rows, rounded, to rows in sorted order
-//   moe_tiles_down      weight * W_down act for a tile's rows, float32, to y[chosen place][token]: the `top` places
+//   gate/up             act(W_gate x) * (W_up x) for a tile's rows, rounded, to rows in sorted order
+//   down                weight * W_down act for a tile's rows, float32, to y[chosen place][token]: the `top` places
 //                       of a token are float32 partial sums that the stream's next norm adds in order
+// each in three kernels by the step's size: moe_few_tiles (up to 512 pairs), moe_tiles_gate_up / moe_tiles_down (up to
+// 4,096), moe_big_tiles (above).
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 
@@ -459,6 +461,74 @@ __global__ __launch_bounds__(256) void moe_tiles_down_kernel(float* __restrict__
   }
 }
 
+// The two products for steps of up to 512 pairs (decode steps, small portions), where an expert sees at most a few
+// tokens and its weights are streamed exactly once: a tile is up to 16 rows, and the four wavefronts of a workgroup share
+// one tile of 16 features and take a quarter of k each, leave their sums in LDS, and the first adds them in wavefront
+// order (a wavefront per 16 features and the whole of k was measured against it: 35 + 22 us against 25 + 14 at one
+// token, 85 + 57 against 67 + 39 at eight).  The order of adding is a function of the sizes alone.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_few_tiles_kernel(bf16_t* __restrict__ act_out, float* __restrict__ y,
+                                                            const bf16_t* __restrict__ a_rows, int64_t lda,
+                                                            const bf16_t* __restrict__ w_first, const bf16_t* __restrict__ w_second,
+                                                            const int* __restrict__ order, const float* __restrict__ weights,
+                                                            const int4* __restrict__ tiles, int top, int num_tokens, int K,
+                                                            int N, int act_kind) {
+  __shared__ f32x4 parts[3][2][PAE_WAVE];
+  const int4 tile = tiles[blockIdx.x];  // (expert, first sorted row, rows <= 16, unused)
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int col = lane % 16, kg = lane / 16;
+  const int n0 = blockIdx.y * 16;
+  if (tile.z <= 0 || n0 >= N) return;
+  const int64_t w_row = (int64_t)tile.x * N + min(n0 + col, N - 1);
+  const bf16_t* w1 = w_first + w_row * K + 8 * kg;
+  const bf16_t* w2 = GATED ? w_second + w_row * K + 8 * kg : nullptr;
+  const int sorted = tile.y + (col < tile.z ? col : 0);
+  const bf16_t* a = a_rows + (int64_t)(GATED ? order[sorted] / top : sorted) * lda + 8 * kg;
+  const int steps = K / 32, per = (steps + 3) / 4;
+  const int first = wave * per, last = min(steps, first + per);
+  f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
+  if (first < last) {
+    bf16x8 ca = *reinterpret_cast<const bf16x8*>(a + 32 * first), c1 = *reinterpret_cast<const bf16x8*>(w1 + 32 * first), c2;
+    if (GATED) c2 = *reinterpret_cast<const bf16x8*>(w2 + 32 * first);
+    for (int st = first + 1; st < last; ++st) {
+      const bf16x8 na = *reinterpret_cast<const bf16x8*>(a + 32 * st), n1 = *reinterpret_cast<const bf16x8*>(w1 + 32 * st);
+      bf16x8 n2;
+      if (GATED) n2 = *reinterpret_cast<const bf16x8*>(w2 + 32 * st);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c1, ca, s1, 0, 0, 0);
+      if (GATED) s2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c2, ca, s2, 0, 0, 0);
+      ca = na; c1 = n1;
+      if (GATED) c2 = n2;
+    }
+    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c1, ca, s1, 0, 0, 0);
+    if (GATED) s2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c2, ca, s2, 0, 0, 0);
+  }
+  if (wave > 0) {
+    parts[wave - 1][0][lane] = s1;
+    if (GATED) parts[wave - 1][1][lane] = s2;
+  }
+  __syncthreads();
+  if (wave > 0 || col >= tile.z) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    s1 += parts[w][0][lane];
+    if (GATED) s2 += parts[w][1][lane];
+  }
+  const int n = n0 + 4 * kg;  // a lane holds features n .. n + 3 of the row col
+  if (GATED) {
+    bf16_t* o = act_out + (int64_t)(tile.y + col) * N + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) o[i] = __float2bfloat16(act_of(s1[i], act_kind) * s2[i]);
+  } else {
+    const int pair = order[tile.y + col];
+    const float weight = weights[pair];
+    float* o = y + ((int64_t)(pair % top) * num_tokens + pair / top) * N + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) o[i] = weight * s1[i];
+  }
+}
+
 // The same two products for prompts, where an expert sees hundreds of tokens: a workgroup takes a tile of 128 rows
 // and 128 features with gate and up (or 256 output features of the down product), and its operands pass through LDS:
 // every 64 of k, the 256 threads fetch 128 rows of activations and 256 rows of weights, a whole 128-byte line a row, into
@@ -619,8 +689,16 @@ extern "C" int pae_moe_experts_tiles(float* y, const void* x, int64_t ldx, const
                                                                        weights, (const int4*)tiles, top, num_tokens, hidden, \
                                                                        inter);                                              \
   } while (0)
-  if (tile_rows == 16) MOE_TILES(1, 1, 1);
-  else if (tile_rows == 64) MOE_TILES(4, 2, 4);
+  if (tile_rows == 16) {
+    dim3 up_grid(max_tiles, (inter + 15) / 16), down_grid(max_tiles, (hidden + 15) / 16);
+    PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);
+    moe_few_tiles_kernel<true><<<up_grid, 256, 0, stream>>>((bf16_t*)act, nullptr, (const bf16_t*)x, ldx, (const bf16_t*)gate_w,
+                                                            (const bf16_t*)up_w, order, weights, (const int4*)tiles, top,
+                                                            num_tokens, hidden, inter, act_kind);
+    moe_few_tiles_kernel<false><<<down_grid, 256, 0, stream>>>(nullptr, y, (const bf16_t*)act, inter, (const bf16_t*)down_w,
+                                                               nullptr, order, weights, (const int4*)tiles, top, num_tokens,
+                                                               inter, hidden, act_kind);
+  } else if (tile_rows == 64) MOE_TILES(4, 2, 4);
   else {
     dim3 up_grid(max_tiles, (inter + 127) / 128), down_grid(max_tiles, (hidden + 255) / 256);
     PAE_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "experts: widths %d, %d exceed the grid", hidden, inter);
