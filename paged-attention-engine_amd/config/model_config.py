@@ -111,9 +111,10 @@ class MixerSpec(PartSpec):
 
     @property
     def plain(self) -> bool:
-        """The reference's attention and nothing more: what the matrix-core kernels compute."""
+        """The reference's attention and nothing more, with heads in multiples of 16 up to 256: what the kernels of
+        the first path compute (any other head size takes the path for value widths, caps and sinks)."""
         return (self.value_dim in (None, self.head_dim) and self.softcap is None and not self.sinks
-                and self.qk_norm is None and not self.convolved)
+                and self.qk_norm is None and not self.convolved and self.head_dim % 16 == 0 and 16 <= self.head_dim <= 256)
 
     @property
     def convolved(self) -> bool:

@@ -93,8 +93,6 @@ class PagedAttention(Part):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
             raise ValueError(f"{spec.num_heads} query heads over {spec.num_kv_heads} key/value heads")
-        if spec.plain and (spec.head_dim % 16 or not 16 <= spec.head_dim <= 256):
-            raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of 16 up to 256")
         if not spec.plain and not (0 < spec.head_dim <= 1024 and 0 < spec.v_dim <= 256):
             raise ValueError(f"head_dim {spec.head_dim} / value_dim {spec.v_dim}: the attention kernel takes up to 1024 / 256")
         if spec.qk_norm not in (None, "projection", "head"):

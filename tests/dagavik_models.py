@@ -91,10 +91,11 @@ Y = {"architecture": "Dagavik", "vocab": 400, "width": 128, "norm": {"eps": 1e-5
          layer(parallel(window(4, 4, 32, 32, 0.25, size=16, rot_dims=16, base=100.0), 2, 64, 64, 12.0, 0.5, 1.5)),
          layer(latent(8, 16, 16, 64, 0.3, kv_from=0), moe(64, 8, 2, 2.0, 2, 1)),
      ]}
-# Z: nothing is a multiple of four; a window of one token (a token sees itself alone)
+# Z: nothing is a multiple of four; values as wide as keys at a width the first attention path does not take; a window
+# of one token (a token sees itself alone)
 Z = {"architecture": "Dagavik", "vocab": 97, "width": 90, "norm": {"eps": 1e-5},
      "embedding": {"bigram": {"buckets": 7, "mul_prev": 1000003, "mul_cur": 999983}}, "layers": [
-         layer(parallel(window(3, 3, 22, 18, 0.3, size=1, rot_dims=10, base=50.0), 3, 10, 14, 6.0, 1.1, 0.9), moe(14, 6, 1, 3.0, 3, 1)),
+         layer(parallel(window(3, 3, 22, 22, 0.3, size=1, rot_dims=10, base=50.0), 3, 10, 14, 6.0, 1.1, 0.9), moe(14, 6, 1, 3.0, 3, 1)),
          layer(delta(3, 1, 10, 14, 3, 6, 10), moe(10, 7, 3, 0.5)),
          layer(latent(3, 10, 14, 22, 0.35), moe(14, 6, 1, 3.0, 3, 1)),
      ]}
