@@ -51,15 +51,29 @@ class FrequencyRamp:
 
 
 @dataclass(frozen=True)
+class WavelengthRamp:
+    """Frequencies of a rotation stretched by wavelength (the scaling of Llama 3.1): with l = 2 pi / f a pair's
+    wavelength, a pair with l < original / high keeps its frequency, one with l > original / low has it divided
+    by `factor`, and between the two the frequencies f / factor and f are blended linearly in original / l:
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low).  Cosines and sines keep their size."""
+
+    factor: float
+    original: float
+    low: float
+    high: float
+
+
+@dataclass(frozen=True)
 class PositionSpec(PartSpec):
     """Rotation of query and key by absolute position; `rotary_dim` leading
     features of each head are rotated in pairs: (i, i + rotary_dim/2) for kind
-    "neox_rope", (2i, 2i + 1) for kind "interleaved_rope" (which also takes a `ramp`)."""
+    "neox_rope", (2i, 2i + 1) for kind "interleaved_rope" (which also takes a `ramp`:
+    a `FrequencyRamp` or a `WavelengthRamp`)."""
 
     rotary_dim: int = 0
     theta: float = 10000.0
     kind: str = "neox_rope"
-    ramp: Optional[FrequencyRamp] = None
+    ramp: Optional[object] = None
 
 
 @dataclass(frozen=True)
@@ -91,7 +105,10 @@ class MixerSpec(PartSpec):
     softcap: Optional[float] = None      # scores become softcap * tanh(score / softcap)
     sinks: bool = False                  # one learned number per query head joins the softmax's denominator
     sink_name: str = "sinks"
-    qk_norm: Optional[str] = None        # "projection": RMS norm over the whole q and the whole k projection
+    fixed_sink: Optional[float] = None   # instead of learned sinks: every head's sink is this number (0: the
+                                         # denominator is one larger than the sum of exponentials); no tensor
+    qk_norm: Optional[str] = None        # "projection": RMS norm over the whole q and the whole k projection;
+                                         # "per_head": over each head, with one weight [head_dim] shared by the heads
     qk_norm_eps: float = 1e-6
     q_norm_name: str = "q_norm.weight"
     k_norm_name: str = "k_norm.weight"
@@ -114,7 +131,7 @@ class MixerSpec(PartSpec):
         """The reference's attention and nothing more, with heads in multiples of 16 up to 256: what the kernels of
         the first path compute (any other head size takes the path for value widths, caps and sinks)."""
         return (self.value_dim in (None, self.head_dim) and self.softcap is None and not self.sinks
-                and self.qk_norm is None and not self.convolved and self.head_dim % 16 == 0 and 16 <= self.head_dim <= 256)
+                and self.fixed_sink is None and self.qk_norm is None and not self.convolved and self.head_dim % 16 == 0 and 16 <= self.head_dim <= 256)
 
     @property
     def convolved(self) -> bool:
@@ -219,6 +236,34 @@ class MatrixMemorySpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class LinearAttentionSpec(PartSpec):
+    """Gated linear attention: a recurrent mixer with one state matrix [key_dim, value_dim] per head that decays,
+    per token, by a factor of its own for every key channel: S <- diag(a_t) S + k_t v_t^T, o_t = S^T q_t, with
+    a = sigmoid(z)^(1 / decay_temperature) and z through two narrow products with `decay_rank` features between
+    and a bias.  q is multiplied by key_dim^-1/2; o is RMS-normed per head with a weight [value_dim] shared by the
+    heads, gated by `gate_activation`(W_g h) and projected out."""
+
+    hidden_size: int = 0
+    num_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    decay_rank: int = 0
+    decay_temperature: float = 1.0
+    norm_eps: float = 1e-6
+    gate_activation: str = "silu"    # or "sigmoid"
+    kind: str = "gated_linear_attention"
+    q_name: str = "q"
+    k_name: str = "k"
+    v_name: str = "v"
+    gate_name: str = "g"
+    decay_name: str = "a"            # the two narrow products are <decay_name>1 and <decay_name>2, the bias <decay_name>2<bias_suffix>
+    o_name: str = "o"
+    norm_name: str = "norm"
+    bias_suffix: str = ".b"
+    weight_suffix: str = ""
+
+
+@dataclass(frozen=True)
 class SideBySideSpec(PartSpec):
     """Two mixers that read the same input; the result is left_scale * left + right_scale * right.  Their
     tensors lie below `left_prefix` and `right_prefix` of the mixer's own prefix."""
@@ -249,6 +294,8 @@ class ExpertsSpec(PartSpec):
     activation: str = "silu"
     kind: str = "experts"
     router_name: str = "router"
+    choice_bias_name: Optional[str] = None  # a tensor [experts] added to the scores where experts are chosen (the
+                                            # weights stay the scores themselves); None: no such tensor
     expert_prefix: str = "e"   # expert j's tensors lie below <expert_prefix><j>.
     gate_name: str = "gate"
     up_name: str = "up"
@@ -266,6 +313,25 @@ class PairEmbeddingSpec:
     buckets: int
     mul_prev: int
     mul_cur: int
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A layer's own input from the token: the layer reads `dim` columns, from `first_column` on, of a second
+    token table `table_name` [vocab, table_width] shared by the layers, e = table[token][first_column : + dim], and
+    adds  N(W_proj (act(W_gate x) * e))  to the stream x it has just written, N an RMS norm with a plain weight."""
+
+    table_name: str
+    table_width: int
+    first_column: int
+    dim: int
+    vocab_size: int
+    eps: float
+    activation: str = "gelu_tanh"
+    gate_name: str = "gate"
+    proj_name: str = "proj"
+    norm_name: str = "norm"
+    weight_suffix: str = ""
 
 
 @dataclass(frozen=True)
@@ -304,6 +370,14 @@ class LayerSpec:
     streams: int = 1
     connection_prefixes: Optional[Tuple[str, str]] = None
     layer_scale_names: Optional[Tuple[str, str]] = None
+    # arrangement "sandwich": a norm before and a norm after each sublayer, x <- x + norm_out(sublayer(norm(x)));
+    # the norms after, with their prefixes, and what the token itself feeds the layer after its feed-forward
+    mixer_out_norm: Optional[PartSpec] = None
+    feed_forward_out_norm: Optional[PartSpec] = None
+    mixer_out_norm_prefix: str = ""
+    feed_forward_out_norm_prefix: str = ""
+    token_side: Optional[TokenSideSpec] = None
+    token_side_prefix: str = "side."
 
 
 @dataclass(frozen=True)
@@ -313,10 +387,12 @@ class ScheduleEntry:
     `layer` indexes `ModelPlan.layers` (a layer may be named by several
     entries: its weights are then shared while each entry keeps a cache of its
     own).  `cache_from` names an earlier *entry* whose cache this entry reads
-    instead of writing one."""
+    instead of writing one.  `add_embedding`: before this stop runs, the embedding's output (the
+    stream as it was before the first stop) is added to the stream once more."""
 
     layer: int
     cache_from: Optional[int] = None
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -341,6 +417,7 @@ class ModelPlan:
     logit_softcap: Optional[float] = None   # ... and then, with a cap c, become c * tanh(logits / c)
     streams: int = 1                        # copies the residual stream is kept in (blocks of arrangement "hyper")
     pair_embedding: Optional[PairEmbeddingSpec] = None  # a hashed table of token pairs added to the embedding
+    position_table_name: Optional[str] = None  # a learned row per position [max_positions, hidden], added unscaled
     extra: Mapping[str, Any] = field(default_factory=dict)
 
     def __post_init__(self) -> None:
@@ -356,6 +433,10 @@ class ModelPlan:
                 raise ConfigError(f"layer {i} keeps {layer.streams} copies of the stream, the model {self.streams}")
             if layer.streams != 1 and layer.arrangement != "hyper":
                 raise ConfigError(f"layer {i}: only the arrangement 'hyper' keeps several copies of the stream")
+        if self.position_table_name is not None and not self.max_positions:
+            raise ConfigError("a table of learned positions needs max_positions, its number of rows")
+        if self.schedule and self.schedule[0].add_embedding:
+            raise ConfigError("the first stop of the schedule cannot add the embedding's output again")
         if self.logit_softcap is not None and not self.logit_softcap > 0:
             raise ConfigError(f"logit_softcap must be positive, got {self.logit_softcap}")
 

@@ -98,12 +98,13 @@ int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q, int64_t q
                          const int* block_tables, int max_blocks, int bs, int H, int kd, int C, float scale, int window,
                          int chunked, float* part_acc, float* part_ml, const float* sinks, hipStream_t stream);
 int pae_latent_attn_split();
-// rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
+// rows [q | k | v]: RMS norm of q and of k over the whole projection, or head by head with one weight that the
+// heads share (`per_head`; weights null: none), rotation, cache write
 int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
                              const void* q_w, const void* k_w, int w_is_f32, float eps, int rot, int interleaved,
                              const float* cos_sin, float magnitude, const int* positions, const int* tok_seq,
                              const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv,
-                             hipStream_t stream);
+                             int per_head, hipStream_t stream);
 // blocks that normalise a branch's output: see branch_norm.hip
 int pae_rows_from_residual(int dtype, void* out, const float* residual, int64_t n, hipStream_t stream);
 int pae_norm_scale_add(int dtype, float* residual, const void* y, int parts, int64_t part_stride, const void* weight,
@@ -134,11 +135,28 @@ int pae_sum_norm2(int dtype, float* residual, int num_terms, const void* const* 
                   const int* term_parts, const int64_t* term_part_stride, const float* term_scale, const void* w1,
                   int w1_is_f32, const void* w2, int w2_is_f32, float eps, const int* rows, void* out1, void* out2,
                   int num_rows, int hidden, int write_residual, hipStream_t stream);
+// a sublayer's output joins the stream through the norm after it; the norm before the next sublayer: see sandwich_norm.hip
+int pae_norm_join(int dtype, float* residual, int num_terms, const void* const* term_ptr, const int* term_is_f32,
+                  const int* term_parts, const int64_t* term_part_stride, const float* term_scale, const void* w_out,
+                  int w_out_is_f32, float eps, const void* w_next, int w_next_is_f32, float eps_next, void* normed,
+                  void* rows, int num_rows, int hidden, hipStream_t stream);
+// gated linear attention over a step's projected rows: see linear_attention.hip
+int pae_linear_attention_step(int dtype, const void* proj, int64_t row_stride, const void* z_in, int64_t z_stride,
+                              const void* z_bias, int bias_is_f32, float tau, const void* gate_in, int64_t gate_stride,
+                              int gate_sigmoid, int num_tokens, int num_seqs, const int* seq_runs, const int* slots, int H,
+                              int D, int V, float* state, int64_t state_slot_stride, const void* norm_w, int w_is_f32,
+                              float norm_eps, float* work, void* out, hipStream_t stream);
+int64_t pae_linear_attention_work_floats(int num_tokens, int H, int D, int V);
+// a learned row per position added to the embedding; a layer's columns of a second token table: see token_inputs.hip
+int pae_embedding_positions(int dtype, float* out, const void* table, const int* ids, const void* rows,
+                            const int* positions, int num_tokens, int hidden, int vocab, float scale, hipStream_t stream);
+int pae_token_gate(int dtype, void* out, const void* gate, int64_t gate_stride, const void* columns, const int* ids,
+                   int num_tokens, int dim, int kind, hipStream_t stream);
 // float32 sums of a few output features from rows of either type: see moe.hip
 int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* bias,
                     int b_is_f32, int M, int N, int K, hipStream_t stream);
 int pae_moe_route(const float* logits, int num_tokens, int experts, int groups, int keep, int top, float scale,
-                  int* chosen, float* weights, hipStream_t stream);
+                  const float* choice_bias, int* chosen, float* weights, hipStream_t stream);
 int pae_moe_gate_up(int dtype, void* act, const void* x, int64_t ldx, const void* gate_w, const void* up_w,
                     const int* chosen, int num_tokens, int top, int hidden, int inter, int act_kind, hipStream_t stream);
 int pae_moe_tile_rows(int pairs);

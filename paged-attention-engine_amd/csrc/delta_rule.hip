@@ -366,6 +366,22 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float*
   }
 }
 
+// The gated norm over a step's read-outs `o` [T][H][V], for mixers that share it (linear_attention.hip).
+int pae_launch_gated_norm(int dtype, const float* o, const void* gates, int64_t gate_stride, int gate_sigmoid,
+                          const void* weight, int w_is_f32, float eps, int num_tokens, int H, int V, void* out,
+                          hipStream_t stream) {
+  dim3 grid(num_tokens, H);
+  if (dtype == PAE_F32)
+    delta_gated_norm_kernel<float><<<grid, PAE_WAVE, 0, stream>>>(o, (const float*)gates, gate_stride, gate_sigmoid, weight,
+                                                                  w_is_f32, eps, H, V, (float*)out);
+  else if (dtype == PAE_BF16)
+    delta_gated_norm_kernel<bf16_t><<<grid, PAE_WAVE, 0, stream>>>(o, (const bf16_t*)gates, gate_stride, gate_sigmoid, weight,
+                                                                   w_is_f32, eps, H, V, (bf16_t*)out);
+  else
+    return pae_fail("gated norm: unknown dtype code %d", dtype);
+  return 0;
+}
+
 static int lanes_per_column(int D, int R);
 void pae_launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
                            const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,

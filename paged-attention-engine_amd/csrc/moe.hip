@@ -6,7 +6,8 @@
 //                   equal groups of neighbours, a group's score is its largest score, only experts of the
 //                   `keep` best groups can be chosen; the `top` largest scores among those are chosen,
 //                   and their weights are the scores times `scale` (not renormalised).  Of equal
-//                   scores the lower index wins.  One wavefront a token.
+//                   scores the lower index wins.  With a `choice_bias` [E], experts and groups are compared
+//                   by score + bias, while the weights stay the scores themselves.  One wavefront a token.
 //   moe_gate_up     for every (token, chosen expert): act(W_gate x) * (W_up x), rounded to the activation type
 //   moe_down        for every token: sum over its chosen experts of weight * W_down act, float32
 //
@@ -87,11 +88,12 @@ extern "C" int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A
 #define MOE_MAX_PER_LANE 16  // experts a lane holds: up to 1,024 experts
 
 __global__ __launch_bounds__(PAE_WAVE) void moe_route_kernel(const float* __restrict__ logits, int E, int groups, int keep,
-                                                             int top, float scale, int* __restrict__ chosen,
-                                                             float* __restrict__ weights) {
-  extern __shared__ float lds[];  // [E] scores, [groups] group scores
+                                                             int top, float scale, const float* __restrict__ choice_bias,
+                                                             int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float lds[];  // [E] scores, [groups] group scores, and with a bias [E] what experts are compared by
   float* score = lds;
   float* group_score = lds + E;
+  float* rank = choice_bias ? group_score + groups : score;
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
   const float* z = logits + t * E;
@@ -105,11 +107,13 @@ __global__ __launch_bounds__(PAE_WAVE) void moe_route_kernel(const float* __rest
     sum += p;
   }
   sum = wave_sum(sum);
+  if (choice_bias)
+    for (int e = lane; e < E; e += PAE_WAVE) rank[e] = score[e] / sum + choice_bias[e];
   __syncthreads();
   const int per_group = E / groups;
   for (int g = lane; g < groups; g += PAE_WAVE) {
     float best = -INFINITY;
-    for (int j = 0; j < per_group; ++j) best = fmaxf(best, score[g * per_group + j]);
+    for (int j = 0; j < per_group; ++j) best = fmaxf(best, rank[g * per_group + j]);
     group_score[g] = best;
   }
   __syncthreads();
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(PAE_WAVE) void moe_route_kernel(const float* __rest
       const float gs = group_score[g];
       int before = 0;
       for (int o = 0; o < groups; ++o) before += (group_score[o] > gs || (group_score[o] == gs && o < g)) ? 1 : 0;
-      if (before < keep) mine[j] = score[e];
+      if (before < keep) mine[j] = rank[e];
     }
   }
   for (int r = 0; r < top; ++r) {
@@ -147,7 +151,7 @@ __global__ __launch_bounds__(PAE_WAVE) void moe_route_kernel(const float* __rest
     }
     if (lane == 0) {
       chosen[t * top + r] = at;
-      weights[t * top + r] = best / sum * scale;
+      weights[t * top + r] = score[at] / sum * scale;
     }
 #pragma unroll
     for (int j = 0; j < MOE_MAX_PER_LANE; ++j)
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(PAE_WAVE) void moe_route_kernel(const float* __rest
 }
 
 extern "C" int pae_moe_route(const float* logits, int num_tokens, int experts, int groups, int keep, int top, float scale,
-                             int* chosen, float* weights, hipStream_t stream) {
+                             const float* choice_bias, int* chosen, float* weights, hipStream_t stream) {
   PAE_REQUIRE(experts > 0 && experts <= PAE_WAVE * MOE_MAX_PER_LANE, "routing: %d experts (1..%d)", experts,
               PAE_WAVE * MOE_MAX_PER_LANE);
   PAE_REQUIRE(groups > 0 && experts % groups == 0 && keep > 0 && keep <= groups, "routing: %d groups of %d experts, %d kept",
@@ -164,8 +168,8 @@ extern "C" int pae_moe_route(const float* logits, int num_tokens, int experts, i
   PAE_REQUIRE(top > 0 && top <= keep * (experts / groups), "routing: %d experts chosen of %d that can be", top,
               keep * (experts / groups));
   if (num_tokens <= 0) return 0;
-  moe_route_kernel<<<num_tokens, PAE_WAVE, (size_t)(experts + groups) * sizeof(float), stream>>>(
-      logits, experts, groups, keep, top, scale, chosen, weights);
+  moe_route_kernel<<<num_tokens, PAE_WAVE, (size_t)(experts + groups + (choice_bias ? experts : 0)) * sizeof(float), stream>>>(
+      logits, experts, groups, keep, top, scale, choice_bias, chosen, weights);
   return pae_check_launch("moe_route");
 }
 

@@ -56,6 +56,8 @@ def expected_tensors(plan: ModelPlan) -> Dict[str, Tuple[int, ...]]:
         out[plan.head_name] = (plan.vocab_size, plan.hidden_size)
     if plan.pair_embedding is not None:
         out[plan.pair_embedding.name] = (plan.pair_embedding.buckets + 1, plan.hidden_size)
+    if plan.position_table_name is not None:
+        out[plan.position_table_name] = (plan.max_positions, plan.hidden_size)
     return out
 
 
@@ -87,6 +89,10 @@ class Model:
         self.pair_table = None
         if plan.pair_embedding is not None:
             self.pair_table = weights[plan.pair_embedding.name].to(device=self.device, dtype=self.dtype).contiguous()
+        self.position_table = None
+        if plan.position_table_name is not None:
+            self.position_table = weights[plan.position_table_name].to(device=self.device, dtype=self.dtype).contiguous()
+        self._embedding_joins_again = any(entry.add_embedding for entry in plan.schedule)
         for block in self.blocks:
             block.bind(weights)
         self.final_norm.bind(plan.final_norm_prefix, weights)
@@ -171,14 +177,24 @@ class Model:
     def max_program_phases(self) -> int:
         return 8 * len(self.plan.schedule) + 8
 
-    def _run_blocks(self, ctx: StepContext, stream: ResidualStream, first_norms) -> None:
-        for index, entry in enumerate(self.plan.schedule):
+    def _run_blocks(self, ctx: StepContext, stream: ResidualStream, first_norms, embedded=None) -> None:
+        schedule = self.plan.schedule
+        for index, entry in enumerate(schedule):
             ctx.entry = index
             ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
             ctx.writes_cache = entry.cache_from is None
+            if entry.add_embedding:
+                # the embedding's output joins the stream once more before this stop (a pass over shared layers)
+                if stream.pending is not None or stream.owed is not None or stream.copies != 1 or stream.prepared is not None:
+                    raise ValueError(f"stop {index}: the embedding's output can only join a plain stream with nothing pending")
+                K.residual_add(stream.residual, embedded)
+                stream.rows = None
             stream.next_norm = first_norms[index + 1]
-            after = self.plan.schedule[index + 1].layer if index + 1 < len(self.plan.schedule) else None
-            stream.rows_wanted_next = after is not None and getattr(self.blocks[after], "reads_stream_rows", False)
+            after = schedule[index + 1].layer if index + 1 < len(schedule) else None
+            stream.rows_wanted_next = (after is not None and getattr(self.blocks[after], "reads_stream_rows", False)
+                                       and not schedule[index + 1].add_embedding)
+            stream.prepared_wanted_next = (after is not None and getattr(self.blocks[after], "takes_prepared_norm", False)
+                                           and not schedule[index + 1].add_embedding)
             self.blocks[entry.layer].forward(ctx, stream)
             if self.residual_tap is not None:
                 self.residual_tap(index, stream)
@@ -198,11 +214,19 @@ class Model:
             stream = ResidualStream(torch.empty((T, copies * H), dtype=torch.float32, device=self.device))
             stream.copies = copies
         stream.sum_weights = self._sum_weights
+        ctx.token_ids = token_ids
         # the norm that reads the stream first at every stop (and the final norm after the last)
         first_norms = [getattr(self.blocks[entry.layer], "mixer_norm", None) for entry in plan.schedule] + [self.final_norm]
         entry_fold = getattr(self.blocks[plan.schedule[0].layer], "entry_fold", None) if plan.schedule and T else None
-        fold = entry_fold(T) if entry_fold is not None and plan.pair_embedding is None else None
-        if fold is not None:
+        own_kernel = plan.pair_embedding is not None or self.position_table is not None
+        fold = entry_fold(T) if entry_fold is not None and not own_kernel else None
+        if self.position_table is not None:
+            if plan.pair_embedding is not None or copies > 1:
+                raise ValueError("a table of learned positions goes with a plain embedding and one copy of the stream")
+            if ctx.q_lens and max(p + n for p, n in zip(ctx.past_lens, ctx.q_lens)) > plan.max_positions:
+                raise ValueError(f"a sequence passes the {plan.max_positions} positions the model has rows for")
+            K.embedding_positions(residual, self.embedding, token_ids, self.position_table, ctx.positions, plan.embedding_scale)
+        elif fold is not None:
             # the first block's norm lets the embedding prepare its rows (see parts.OwedRows)
             norm, weight, eps = fold
             rows = torch.empty((T, H), dtype=torch.bfloat16, device=self.device)
@@ -220,14 +244,19 @@ class Model:
             K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
             if copies > 1:
                 K.hyper_spread(stream.residual, residual, copies)
+        embedded = None
+        if self._embedding_joins_again:
+            if copies > 1:
+                raise ValueError("the embedding's output joins a plain stream, not one kept in copies")
+            embedded = residual.clone()  # the stream as it was before the first stop
         program = ctx.program if fold is not None and self.decode_fusable(ctx) else None
         if program is not None:
             # every block's kernels become phases of one resident kernel, which runs when all are recorded
             with K.recording(program):
-                self._run_blocks(ctx, stream, first_norms)
+                self._run_blocks(ctx, stream, first_norms, embedded)
             program.launch()
         else:
-            self._run_blocks(ctx, stream, first_norms)
+            self._run_blocks(ctx, stream, first_norms, embedded)
         rows = logit_rows.numel()
         if rows == 0:
             return torch.empty((0, plan.vocab_size), dtype=torch.float32, device=self.device)

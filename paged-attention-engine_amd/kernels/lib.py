@@ -72,7 +72,7 @@ def _declare(lib) -> None:
         "pae_gemm_skinny_gated": [P, L, P, L, P, I, I, I, I, P, P, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_paged_attention_capped": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, P],
-        "pae_qk_norm_rotate_store": [I, P, L, I, I, I, I, I, P, P, I, F, I, I, P, F, P, P, P, I, I, P, P, I, P],
+        "pae_qk_norm_rotate_store": [I, P, L, I, I, I, I, I, P, P, I, F, I, I, P, F, P, P, P, I, I, P, P, I, I, P],
         "pae_paged_attention_masked": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, I, P, P, L, I, P],
         "pae_hyper_norm": [I, P, I, P, I, L, P, I, P, P, P, P, I, F, P, P, I, I, I, P],
         "pae_hyper_spread": [P, P, I, I, I, P],
@@ -95,7 +95,11 @@ def _declare(lib) -> None:
         "pae_embedding_pairs": [I, P, P, P, P, P, P, P, P, I, I, I, F, I, I, I, P],
         "pae_sum_norm2": [I, P, I, P, P, P, P, P, P, I, P, I, F, P, P, P, I, I, I, P],
         "pae_project_f32": [I, P, L, P, L, P, P, I, I, I, I, P],
-        "pae_moe_route": [P, I, I, I, I, I, F, P, P, P],
+        "pae_moe_route": [P, I, I, I, I, I, F, P, P, P, P],
+        "pae_norm_join": [I, P, I, P, P, P, P, P, P, I, F, P, I, F, P, P, I, I, P],
+        "pae_linear_attention_step": [I, P, L, P, L, P, I, F, P, L, I, I, I, P, P, I, I, I, P, L, P, I, F, P, P, P],
+        "pae_embedding_positions": [I, P, P, P, P, P, I, I, I, F, P],
+        "pae_token_gate": [I, P, P, L, P, P, I, I, I, P],
         "pae_moe_gate_up": [I, P, P, L, P, P, P, I, I, I, I, I, P],
         "pae_moe_down": [I, P, P, P, P, P, I, I, I, I, P],
         "pae_moe_tile_rows": [I],
@@ -136,6 +140,8 @@ def _declare(lib) -> None:
     lib.pae_delta_rule_work_floats.restype = c_int64
     lib.pae_matrix_memory_work_floats.argtypes = [I, I, I, I]
     lib.pae_matrix_memory_work_floats.restype = c_int64
+    lib.pae_linear_attention_work_floats.argtypes = [I, I, I, I]
+    lib.pae_linear_attention_work_floats.restype = c_int64
 
 
 def _check(code: int) -> None:
@@ -196,6 +202,36 @@ def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: 
     assert ids.dtype == torch.int32 and ids.numel() == T and table.shape[1] == H
     _check(library().pae_embedding(code_of(table.dtype), out.data_ptr(), table.data_ptr(), ids.data_ptr(),
                                    T, H, table.shape[0], float(scale), _stream()))
+
+
+def embedding_positions(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, rows: torch.Tensor,
+                        positions: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t] = scale * table[ids[t]] + rows[positions[t]] as float32: `rows` [max positions, H] holds a learned row
+    per position, added unscaled.  The caller vouches that every position lies within `rows`."""
+    _not_while_recording("embedding_positions")
+    _gpu(out, table, ids, rows, positions)
+    T, H = out.shape
+    assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous() and rows.is_contiguous()
+    assert table.dtype == rows.dtype and table.shape[1] == H == rows.shape[1]
+    for t in (ids, positions):
+        assert t.dtype == torch.int32 and t.numel() == T and t.is_contiguous()
+    _check(library().pae_embedding_positions(code_of(table.dtype), out.data_ptr(), table.data_ptr(), ids.data_ptr(),
+                                             rows.data_ptr(), positions.data_ptr(), T, H, table.shape[0], float(scale),
+                                             _stream()))
+
+
+def token_gate(gate: torch.Tensor, columns: torch.Tensor, ids: torch.Tensor, kind: str) -> torch.Tensor:
+    """[T, dim] in gate's type: act(gate[t]) * columns[ids[t]], `gate` [T, dim] a narrow product of the stream (a view
+    of wider rows will do), `columns` [vocab, dim] a layer's columns of a second token table; float32 inside."""
+    _not_while_recording("token_gate")
+    _gpu(gate, columns, ids)
+    T, dim = gate.shape
+    assert gate.stride(1) == 1 and columns.is_contiguous() and columns.shape[1] == dim and columns.dtype == gate.dtype
+    assert ids.dtype == torch.int32 and ids.numel() == T and ids.is_contiguous() and kind in ACTIVATIONS
+    out = torch.empty((T, dim), dtype=gate.dtype, device=gate.device)
+    _check(library().pae_token_gate(code_of(gate.dtype), out.data_ptr(), gate.data_ptr(), gate.stride(0), columns.data_ptr(),
+                                    ids.data_ptr(), T, dim, ACTIVATIONS[kind], _stream()))
+    return out
 
 
 def logits_finish(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> None:
@@ -1246,9 +1282,10 @@ def qk_norm_rotate_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, vd: int,
                          k_weight: Optional[torch.Tensor], eps: float, rot: int, interleaved: bool,
                          cos_sin: Optional[torch.Tensor], magnitude: float, positions: torch.Tensor,
                          tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
-                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], per_head: bool = False) -> None:
     """Rows [q: nh x hd | k: nkv x hd | v: nkv x vd]: with weights, q and k are each divided by the root
-    mean square of their whole projection and multiplied by the weight; the first `rot` features of
+    mean square of their whole projection and multiplied by the weight (`per_head`: every head by its own root
+    mean square, and the weights are hd numbers that the heads share); the first `rot` features of
     every q and k head are rotated by `cos_sin` times `magnitude` (pairs (2i, 2i+1) if `interleaved`,
     else (i, i + rot/2)); queries are written back in place, keys and values to their cache slots
     (`k_cache` None: nkv must be 0 and nothing is stored)."""
@@ -1261,8 +1298,9 @@ def qk_norm_rotate_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, vd: int,
     _check_cos_sin(cos_sin, rot, T)
     wf = 0
     if q_weight is not None:
-        assert q_weight.numel() == nh * hd and q_weight.is_contiguous()
-        assert nkv == 0 or (k_weight is not None and k_weight.numel() == nkv * hd and k_weight.dtype == q_weight.dtype)
+        assert q_weight.numel() == (hd if per_head else nh * hd) and q_weight.is_contiguous()
+        assert nkv == 0 or (k_weight is not None and k_weight.numel() == (hd if per_head else nkv * hd)
+                            and k_weight.dtype == q_weight.dtype and k_weight.is_contiguous())
         wf = _param(q_weight)[1]
     max_blocks = 0
     if write:
@@ -1275,7 +1313,7 @@ def qk_norm_rotate_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, vd: int,
         code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, vd, _ptr(q_weight), _ptr(k_weight), wf,
         float(eps), rot, 1 if interleaved else 0, _ptr(cos_sin) if rot else None, float(magnitude),
         positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache),
-        1 if write else 0, _stream()))
+        1 if write else 0, 1 if (per_head and q_weight is not None) else 0, _stream()))
 
 
 def rows_from_residual(residual: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -1477,6 +1515,80 @@ def sum_norm2(residual: torch.Tensor, terms, w1: Optional[torch.Tensor], w2: Opt
                                    p2, f2, float(eps), _ptr(rows), _ptr(out1), _ptr(out2), n, H, 1, _stream()))
 
 
+def norm_join(residual: torch.Tensor, terms, w_out: Optional[torch.Tensor], eps: float,
+              w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0, normed: Optional[torch.Tensor] = None,
+              rows: Optional[torch.Tensor] = None) -> None:
+    """A sublayer's output joins the stream through the norm after it: y = sum of scale * term over `terms` (as for
+    `sum_norm2`), residual += y / sqrt(mean(y^2) + eps) * w_out (`w_out` None: residual += y), all float32.  Then,
+    as asked: `normed` = residual / sqrt(mean(residual^2) + eps_next) * w_next, the norm before the next sublayer,
+    and `rows` = the new residual itself, both in the activation type."""
+    _not_while_recording("norm_join")
+    outs = [o for o in (normed, rows) if o is not None]
+    _gpu(residual, w_out, w_next, *outs, *[t for t, _ in terms])
+    T, H = residual.shape
+    assert residual.dtype == torch.float32 and residual.is_contiguous()
+    assert len(terms) <= MAX_SUM_TERMS
+    dtype = outs[0].dtype if outs else None
+    for o in outs:
+        assert o.shape == (T, H) and o.is_contiguous() and o.dtype == dtype
+    assert normed is None or (w_next is not None and w_next.numel() == H)
+    assert w_out is None or w_out.numel() == H
+    ptrs = (c_void_p * MAX_SUM_TERMS)()
+    is_f32, parts = (c_int * MAX_SUM_TERMS)(), (c_int * MAX_SUM_TERMS)()
+    strides, scales = (c_int64 * MAX_SUM_TERMS)(), (c_float * MAX_SUM_TERMS)()
+    for j, (t, scale) in enumerate(terms):
+        assert t.is_contiguous() and tuple(t.shape[-2:]) == (T, H)
+        if t.dim() == 3:
+            assert t.dtype == torch.float32
+        else:
+            assert t.dim() == 2
+            if t.dtype != torch.float32:
+                assert dtype is None or t.dtype == dtype
+                dtype = t.dtype
+        ptrs[j], is_f32[j] = t.data_ptr(), 1 if t.dtype == torch.float32 else 0
+        parts[j], strides[j], scales[j] = (t.shape[0] if t.dim() == 3 else 1), residual.numel(), float(scale)
+    po, fo = _param(w_out)
+    pn, fn = _param(w_next)
+    _check(library().pae_norm_join(code_of(dtype or torch.float32), residual.data_ptr(), len(terms), ptrs, is_f32, parts,
+                                   strides, scales, po, fo, float(eps), pn, fn, float(eps_next), _ptr(normed), _ptr(rows),
+                                   T, H, _stream()))
+
+
+def linear_attention_step(proj: torch.Tensor, decay_in: torch.Tensor, decay_bias: Optional[torch.Tensor], tau: float,
+                          gate: torch.Tensor, out: torch.Tensor, seq_runs: torch.Tensor, slots: torch.Tensor,
+                          state: torch.Tensor, norm_w: torch.Tensor, H: int, D: int, V: int, norm_eps: float,
+                          gate_activation: str = "silu") -> None:
+    """Gated linear attention over a step's rows.  `proj` [T, >= 2HD + HV] holds per token [q | k | v]; `decay_in`
+    [T, HD] and `gate` [T, HV] are views of rows in proj's type; `decay_bias` [HD] joins the decay's input in float32,
+    and the decay is sigmoid(.)^(1 / tau) per head and key channel.  `seq_runs` int32 [S, 4] = (first row, rows, tokens
+    before, 0) per sequence; `slots` int32 [S]; `state` float32 [slots, H, V, D] is the requests' state, read and
+    moved on; `out` [T, H * V] receives the read-out, normed over V with `norm_w` [V] and gated, in proj's type."""
+    _not_while_recording("linear_attention_step")
+    _gpu(proj, decay_in, decay_bias, gate, out, seq_runs, slots, state, norm_w)
+    T, S = proj.shape[0], seq_runs.shape[0]
+    assert gate_activation in ("silu", "sigmoid")
+    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= 2 * H * D + H * V
+    for view, width in ((decay_in, H * D), (gate, H * V)):
+        assert view.dim() == 2 and view.shape == (T, width) and view.dtype == proj.dtype and view.stride(1) == 1
+    assert out.shape == (T, H * V) and out.is_contiguous() and out.dtype == proj.dtype
+    assert slots.dtype == torch.int32 and slots.numel() >= S and slots.is_contiguous()
+    assert seq_runs.dtype == torch.int32 and seq_runs.shape == (S, 4) and seq_runs.is_contiguous()
+    assert seq_runs.data_ptr() % 16 == 0
+    assert state.dtype == torch.float32 and tuple(state.shape[1:]) == (H, V, D) and state[0].is_contiguous()
+    assert norm_w.numel() == V and norm_w.is_contiguous()
+    if decay_bias is not None:
+        assert decay_bias.numel() == H * D and decay_bias.is_contiguous()
+    wp, wf = _param(norm_w)
+    bp, bf = _param(decay_bias)
+    lib = library()
+    work = torch.empty(lib.pae_linear_attention_work_floats(T, H, D, V), dtype=torch.float32, device=proj.device)
+    _check(lib.pae_linear_attention_step(
+        code_of(proj.dtype), proj.data_ptr(), proj.stride(0), decay_in.data_ptr(), decay_in.stride(0), bp, bf, float(tau),
+        gate.data_ptr(), gate.stride(0), 1 if gate_activation == "sigmoid" else 0, T, S, seq_runs.data_ptr(),
+        slots.data_ptr(), H, D, V, state.data_ptr(), state.stride(0), wp, wf, float(norm_eps), work.data_ptr(),
+        out.data_ptr(), _stream()))
+
+
 def project_f32(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 [M, N] = a [M, K] w[N, K]^T (+ bias), summed in float32 from operands of either type: for the few
     output features whose sums must not pass the activation type (router and gate logits)."""
@@ -1493,18 +1605,22 @@ def project_f32(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
-def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int, scale: float):
+def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int, scale: float,
+              choice_bias: Optional[torch.Tensor] = None):
     """(chosen int32 [T, top], weights float32 [T, top]) from router logits float32 [T, E]: scores are the softmax
     over all experts; only experts of the `keep` best of `groups` equal groups of neighbours (a group's score is
-    its largest) can be chosen; the weights are the chosen scores times `scale`."""
+    its largest) can be chosen; the weights are the chosen scores times `scale`.  With `choice_bias` (float32 [E])
+    experts and groups are compared by score + bias; the weights stay the scores."""
     _not_while_recording("moe_route")
-    _gpu(logits)
+    _gpu(logits, choice_bias)
     T, E = logits.shape
     assert logits.dtype == torch.float32 and logits.is_contiguous()
+    if choice_bias is not None:
+        assert choice_bias.dtype == torch.float32 and choice_bias.numel() == E and choice_bias.is_contiguous()
     chosen = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     _check(library().pae_moe_route(logits.data_ptr(), T, E, int(groups), int(keep), int(top), float(scale),
-                                   chosen.data_ptr(), weights.data_ptr(), _stream()))
+                                   _ptr(choice_bias), chosen.data_ptr(), weights.data_ptr(), _stream()))
     return chosen, weights
 
 

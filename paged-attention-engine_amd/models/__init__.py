@@ -1,2 +1,2 @@
 """Architectures.  Importing this package registers every one of them."""
-from . import dagavik, danonex, qwen2, ritalorn  # noqa: F401
+from . import dagavik, danonex, qwen2, ritalorn, zikezen  # noqa: F401

@@ -21,7 +21,10 @@ Beyond the reference's attention, each switched by the spec and absent when it s
 values of a width of their own (`value_dim`), an RMS norm of the whole query projection and of the
 whole key projection before the rotation (`qk_norm = "projection"`), scores capped by
 softcap * tanh(score / softcap), and a learned sink per query head that joins the softmax's
-denominator as exp(sink) without a key or a value (`sinks`).  A spec with any of them takes the
+denominator as exp(sink) without a key or a value (`sinks`), or one number that is every head's sink
+(`fixed_sink`: with 0 the denominator is one larger than the sum of exponentials), or an RMS norm of
+every query and key head by itself with one weight that the heads share (`qk_norm = "per_head"`).
+A spec with any of them takes the
 path `_forward_wide`: the projection, then one kernel that norms, rotates and stores, then the
 attention kernel that knows caps, sinks and value widths.
 
@@ -95,12 +98,15 @@ class PagedAttention(Part):
             raise ValueError(f"{spec.num_heads} query heads over {spec.num_kv_heads} key/value heads")
         if not spec.plain and not (0 < spec.head_dim <= 1024 and 0 < spec.v_dim <= 256):
             raise ValueError(f"head_dim {spec.head_dim} / value_dim {spec.v_dim}: the attention kernel takes up to 1024 / 256")
-        if spec.qk_norm not in (None, "projection", "head"):
-            raise ValueError(f"qk_norm '{spec.qk_norm}' is not known (known: projection, head)")
+        if spec.qk_norm not in (None, "projection", "head", "per_head"):
+            raise ValueError(f"qk_norm '{spec.qk_norm}' is not known (known: projection, head, per_head)")
+        if spec.sinks and spec.fixed_sink is not None:
+            raise ValueError("an attention has learned sinks or one fixed sink, not both")
         if spec.mask not in ("window", "chunk"):
             raise ValueError(f"mask '{spec.mask}' is not known (known: window, chunk)")
         if spec.convolved:
-            if spec.position is not None or spec.qk_norm == "projection" or spec.sinks or spec.softcap:
+            if (spec.position is not None or spec.qk_norm in ("projection", "per_head") or spec.sinks or spec.softcap
+                    or spec.fixed_sink is not None):
                 raise ValueError("an attention with convolutions, per-head norms, chunks, distance bias or a gate "
                                  "takes no rotation, projection norm, sinks or cap")
             if spec.conv_taps is not None and not 1 <= spec.conv_taps <= 64:
@@ -196,7 +202,10 @@ class PagedAttention(Part):
                prefix + s.k_name + s.weight_suffix: (s.num_kv_heads * s.head_dim, s.hidden_size),
                prefix + s.v_name + s.weight_suffix: (s.num_kv_heads * s.v_dim, s.hidden_size),
                prefix + s.o_name + s.weight_suffix: (s.hidden_size, s.num_heads * s.v_dim)}
-        if s.qk_norm:
+        if s.qk_norm == "per_head":
+            out[prefix + s.q_norm_name] = ScaleShape((s.head_dim,))
+            out[prefix + s.k_norm_name] = ScaleShape((s.head_dim,))
+        elif s.qk_norm:
             out[prefix + s.q_norm_name] = ScaleShape((s.num_heads * s.head_dim,))
             out[prefix + s.k_norm_name] = ScaleShape((s.num_kv_heads * s.head_dim,))
         if s.sinks:
@@ -249,6 +258,8 @@ class PagedAttention(Part):
             self.k_norm = self.vector(weights[prefix + s.k_norm_name])
         if s.sinks:  # sinks enter the softmax, which is float32
             self.sinks = weights[prefix + s.sink_name].to(device=self.device, dtype=torch.float32).contiguous()
+        elif s.fixed_sink is not None:
+            self.sinks = torch.full((s.num_heads,), float(s.fixed_sink), dtype=torch.float32, device=self.device)
 
     def _project_encode_store(self, ctx, x, k_cache, v_cache, table):
         """Queries (and, at a stop that owns its cache, keys and values) of the step's tokens:
@@ -307,7 +318,7 @@ class PagedAttention(Part):
                                s.qk_norm_eps, rot, bool(getattr(self.position, "interleaved", False)), cos_sin,
                                float(getattr(self.position, "magnitude", 1.0)), ctx.positions,
                                ctx.tok_seq if nkv else None, table if nkv else None, ctx.cache.block_size,
-                               k_cache, v_cache)
+                               k_cache, v_cache, per_head=s.qk_norm == "per_head")
         attn = torch.empty((qkv.shape[0], s.num_heads * s.v_dim), dtype=qkv.dtype, device=qkv.device)
         work = ctx.memo.get(WORK_LISTS) if self._matrix_cores(ctx.cache.block_size) else None
         attend_paged(attn, qkv, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, work, s.num_heads,

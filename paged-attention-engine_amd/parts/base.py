@@ -93,6 +93,11 @@ class ResidualStream:
         self.copies = 1
         self.join: Optional["StreamJoin"] = None
         self.sum_weights: Optional[torch.Tensor] = None
+        # for blocks that hand the next block its first norm's rows: (that norm, the whole stream normed by it),
+        # left by the kernel that last wrote the stream, and whether the block after this one will take them
+        # (set by the model)
+        self.prepared: Optional[tuple] = None
+        self.prepared_wanted_next = False
 
 
 class BranchTerms(list):
@@ -173,6 +178,7 @@ class StepContext:
     # room for the step's layers as one resident kernel (kernels.lib.DecodeProgram), offered by the step
     # function for steps in which every sequence brings one token; None: every kernel is launched by itself
     program: Optional[object] = None
+    token_ids: Optional[torch.Tensor] = None  # int32 [T], set by the model: for parts that read a token table of their own
     # what a part computes once per step for every layer that has the same part (a table of angles,
     # say), under a key of the part's choosing; the step function also leaves here, under
     # `step_lists_key`, the index lists a part asked for (`Part.step_lists`), as int32 device tensors

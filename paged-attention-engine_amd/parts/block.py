@@ -317,6 +317,116 @@ class ParallelBlock:
         stream.pending = terms
 
 
+@register_block("sandwich")
+class SandwichBlock:
+    """A norm before and a norm after each sublayer:
+    x <- x + norm1b(mixer(norm1(x)));  x <- x + norm2b(feed_forward(norm2(x))), and, for a layer whose spec names a
+    `token_side`, x <- x + norm_s(side(x, token)) (see parts/token_side.py).  A layer whose spec names no
+    feed-forward has no second half.  A sublayer's output (a tensor, float32 partial sums, or the `BranchTerms` of
+    mixers side by side) joins the float32 stream in one kernel that norms it, adds it, and writes what reads the
+    stream next: the norm before the next sublayer, the stream itself for the token's input, or, after the layer's
+    last sublayer, the first norm of the block that follows if that block takes it (`stream.prepared`)."""
+
+    takes_prepared_norm = True
+
+    def __init__(self, layer_spec, dtype, device):
+        from .norm import RMSNorm
+        from .token_side import TokenSide
+        self.spec = layer_spec
+        self.dtype = dtype
+        if layer_spec.mixer_out_norm is None:
+            raise ValueError("the arrangement 'sandwich' needs the norm after the mixer (mixer_out_norm)")
+        self.mixer_norm = build_part(NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.mixer = build_part(MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.mixer_out_norm = build_part(NORMS, "norm", layer_spec.mixer_out_norm, dtype, device)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_out_norm = None
+        if layer_spec.feed_forward is not None:
+            if layer_spec.feed_forward_norm is None or layer_spec.feed_forward_out_norm is None:
+                raise ValueError("the arrangement 'sandwich' needs both norms around the feed-forward")
+            self.feed_forward_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
+            self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+            self.feed_forward_out_norm = build_part(NORMS, "norm", layer_spec.feed_forward_out_norm, dtype, device)
+        for norm in (self.mixer_norm, self.mixer_out_norm, self.feed_forward_norm, self.feed_forward_out_norm):
+            if norm is not None and (not isinstance(norm, RMSNorm) or norm.spec.weight_offset):
+                raise ValueError(f"the norm '{norm.spec.kind}' cannot ride in the kernel that joins a sublayer's output "
+                                 "(an RMS norm with a plain weight can)")
+        self.side = None
+        if layer_spec.token_side is not None:
+            self.side = TokenSide(layer_spec.token_side, dtype, device, layer_spec.mixer_norm.size)
+
+    def _named(self):
+        s = self.spec
+        out = [(self.mixer_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix),
+               (self.mixer_out_norm, s.prefix + s.mixer_out_norm_prefix)]
+        if self.feed_forward is not None:
+            out += [(self.feed_forward_norm, s.prefix + s.feed_forward_norm_prefix),
+                    (self.feed_forward, s.prefix + s.feed_forward_prefix),
+                    (self.feed_forward_out_norm, s.prefix + s.feed_forward_out_norm_prefix)]
+        if self.side is not None:
+            out.append((self.side, s.prefix + s.token_side_prefix))
+        return out
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for part, _ in self._named())
+
+    @property
+    def graph_max_rows(self):
+        limits = [part.graph_max_rows for part, _ in self._named() if part.graph_max_rows is not None]
+        return min(limits) if limits else None
+
+    def parts(self):
+        return [part for part, _ in self._named()]
+
+    def tensors(self):
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        return out
+
+    def bind(self, weights):
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+
+    def _join(self, stream: ResidualStream, y, weight, eps: float, next_norm=None, want_rows: bool = False):
+        """x <- x + norm(y) with the norm's `weight` and `eps`; returns (x normed by `next_norm`, x in the activation
+        type), each None unless asked for."""
+        import torch
+        from ..kernels import lib as K
+        terms = y if isinstance(y, BranchTerms) else BranchTerms([(y, 1.0)])
+        new = lambda: torch.empty(stream.residual.shape, dtype=self.dtype, device=stream.residual.device)
+        normed = new() if next_norm is not None else None
+        rows = new() if want_rows else None
+        K.norm_join(stream.residual, terms, weight, eps, next_norm.weight if next_norm is not None else None,
+                    next_norm.spec.eps if next_norm is not None else 0.0, normed, rows)
+        return normed, rows
+
+    def forward(self, ctx, stream: ResidualStream) -> None:
+        if stream.pending is not None or stream.owed is not None or stream.copies != 1:
+            raise ValueError("a block with norms around its sublayers follows one that left the stream in another form")
+        ctx.sink = None
+        prepared, stream.prepared = stream.prepared, None
+        x = prepared[1] if prepared is not None and prepared[0] is self.mixer_norm else self.mixer_norm.forward(stream)
+        # what follows the layer's last sublayer: the next block's first norm, if that block takes prepared rows
+        follows = stream.next_norm if stream.prepared_wanted_next and isinstance(stream.next_norm, type(self.mixer_norm)) \
+            and not stream.next_norm.spec.weight_offset else None
+        has_ff, has_side = self.feed_forward is not None, self.side is not None
+        y = self.mixer.forward(ctx, x)
+        out = self.mixer_out_norm
+        x, rows = self._join(stream, y, out.weight, out.spec.eps,
+                             self.feed_forward_norm if has_ff else (None if has_side else follows),
+                             want_rows=has_side and not has_ff)
+        if has_ff:
+            y = self.feed_forward.forward(ctx, x)
+            out = self.feed_forward_out_norm
+            x, rows = self._join(stream, y, out.weight, out.spec.eps, None if has_side else follows, want_rows=has_side)
+        if has_side:
+            y = self.side.forward(ctx, rows)
+            x, _ = self._join(stream, y, self.side.weight, self.side.eps, follows)
+        if follows is not None:
+            stream.prepared = (follows, x)
+
+
 def build_block(layer_spec, dtype, device):
     if layer_spec.arrangement not in BLOCKS:
         raise KeyError(f"no block arrangement '{layer_spec.arrangement}'; known: {', '.join(sorted(BLOCKS))}")

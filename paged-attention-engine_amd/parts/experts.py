@@ -7,7 +7,8 @@ among those are chosen, and the output is
 
     sum over the chosen e of  (route_scale * s_e) * W_down_e (act(W_gate_e h) * (W_up_e h))
 
-with the weights not renormalised.  Experts have no biases.
+with the weights not renormalised.  Experts have no biases.  A design may add a stored tensor [E] to the scores
+where experts (and groups) are compared (`choice_bias_name`); the weights stay the scores themselves.
 
 The experts' matrices are bound stacked, [E, F, H], [E, F, H] and [E, H, F], so that a kernel finds an
 expert's weights by its index.  Routing is a function of the token alone, and every (token, expert) pair is
@@ -51,6 +52,8 @@ class Experts(Part):
     def tensors(self, prefix):
         s = self.spec
         out = {prefix + s.router_name + s.weight_suffix: (s.num_experts, s.hidden_size)}
+        if s.choice_bias_name is not None:
+            out[prefix + s.choice_bias_name] = (s.num_experts,)
         for e in range(s.num_experts):
             out[self._expert(prefix, e, s.gate_name)] = (s.intermediate_size, s.hidden_size)
             out[self._expert(prefix, e, s.up_name)] = (s.intermediate_size, s.hidden_size)
@@ -60,6 +63,9 @@ class Experts(Part):
     def bind(self, prefix, weights):
         s = self.spec
         self.router = self.matrix(weights[prefix + s.router_name + s.weight_suffix])
+        self.choice_bias = None
+        if s.choice_bias_name is not None:  # it meets the float32 scores
+            self.choice_bias = weights[prefix + s.choice_bias_name].to(device=self.device, dtype=torch.float32).contiguous()
 
         def stacked(name: str, shape) -> torch.Tensor:
             out = torch.empty((s.num_experts, *shape), dtype=self.dtype, device=self.device)
@@ -75,7 +81,7 @@ class Experts(Part):
         s = self.spec
         x = plain_rows(x)
         logits = K.project_f32(x, self.router)
-        chosen, weights = K.moe_route(logits, s.groups, s.groups_kept, s.top, s.route_scale)
+        chosen, weights = K.moe_route(logits, s.groups, s.groups_kept, s.top, s.route_scale, self.choice_bias)
         if self.routing_tap is not None:
             self.routing_tap(chosen, weights)
         return K.moe_experts(x, self.gate, self.up, self.down, chosen, weights, s.activation)

@@ -65,6 +65,8 @@ def ramped_frequencies(rot: int, theta: float, ramp) -> "tuple[torch.Tensor, flo
     freq = theta ** (-2.0 * i / rot)
     if ramp is None:
         return freq.to(torch.float32), 1.0
+    if hasattr(ramp, "low"):
+        return stretched_by_wavelength(freq, ramp).to(torch.float32), 1.0
 
     def index_of(turns: float) -> float:
         return rot * math.log(ramp.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
@@ -74,6 +76,17 @@ def ramped_frequencies(rot: int, theta: float, ramp) -> "tuple[torch.Tensor, flo
     blend = torch.clamp((i - low) / max(high - low, 0.001), 0.0, 1.0)
     freq = freq / ramp.factor * blend + freq * (1.0 - blend)
     return freq.to(torch.float32), 0.1 * math.log(ramp.factor) + 1.0
+
+
+def stretched_by_wavelength(freq: torch.Tensor, ramp) -> torch.Tensor:
+    """The float64 frequencies `freq` stretched by a `WavelengthRamp`: a pair whose wavelength 2 pi / f is below
+    original / high keeps f, one above original / low gets f / factor, and between the two f / factor and f are
+    blended by s = (original / wavelength - low) / (high - low)."""
+    wavelength = 2.0 * math.pi / freq
+    share = (ramp.original / wavelength - ramp.low) / (ramp.high - ramp.low) if ramp.high != ramp.low else torch.ones_like(freq)
+    blended = (1.0 - share) * freq / ramp.factor + share * freq
+    out = torch.where(wavelength > ramp.original / ramp.low, freq / ramp.factor, blended)
+    return torch.where(wavelength < ramp.original / ramp.high, freq, out)
 
 
 @register_position_encoding("interleaved_rope")
