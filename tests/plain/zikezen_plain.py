@@ -29,8 +29,10 @@ import math
 
 import torch
 
-# See tests/plain/danonex_plain.py: with STORAGE set, products read and write values rounded to it.
+# See tests/plain/danonex_plain.py: with STORAGE set, products read and write values rounded to it;
+# with JITTER = (generator, size) their sums are moved at random by that relative size first.
 STORAGE = None
+JITTER = None
 
 
 def stored(x: torch.Tensor) -> torch.Tensor:
@@ -41,6 +43,8 @@ def product(h: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = N
     y = stored(h) @ weight.T
     if bias is not None:
         y = y + bias
+    if JITTER is not None:
+        y = y * (1.0 + JITTER[1] * torch.randn(y.shape, generator=JITTER[0], dtype=y.dtype))
     return stored(y)
 
 
@@ -65,7 +69,7 @@ def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
 
 def embed(W: dict, cfg: dict, tokens, dtype) -> torch.Tensor:
     ids = torch.as_tensor(list(tokens), dtype=torch.long)
-    x = W["embed"].to(dtype)[ids] * float(cfg["embedding"]["scale"])
+    x = W["embed"].to(dtype)[ids] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     return x + W["pos"].to(dtype)[: len(ids)]
 
 
