@@ -138,11 +138,39 @@ def dagavik_shape(shape: dict, layers: int) -> dict:
             "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": out}
 
 
+def zikezen_shape(shape: dict, layers: int) -> dict:
+    """A Zikezen configuration with the layer sizes of the Qwen2.5 shape `shape`, `layers` layer runs in all: the same
+    width, head counts and head size in the attention half of its mixers (values as wide as keys, half of each head
+    rotated with frequencies stretched by wavelength, a window of 2,048, per-head norms, the sink) beside gated
+    linear attention with as many heads of the same size (narrow products of half a head size, a temperature of
+    16); feed-forwards in turn dense, of the shape's width, and routed, 32 experts of a quarter of that width with
+    four a token, so that a token's feed-forward always does the dense one's arithmetic; the second and third layer
+    run twice (so the model has two layers fewer than runs); a second token table of 64 columns a layer; learned
+    positions; a logit cap; the same vocabulary."""
+    heads, kv, hd = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    mixer = {"left": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 2048},
+                      "rot": {"base": float(shape["rope_theta"]), "dims": hd // 2,
+                              "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+             "right": {"heads": heads, "dim": hd, "vdim": hd, "tau": 16.0, "decay_rank": hd // 2},
+             "left_scale": 0.7, "right_scale": 0.7}
+    dense = {"kind": "dense", "ff": shape["intermediate_size"]}
+    moe = {"kind": "moe", "expert": {"ff": shape["intermediate_size"] // 4 // 8 * 8}, "router": {"experts": 32, "top": 4}}
+    looped = layers >= 4
+    count = layers - 2 if looped else layers
+    out = {"architecture": "Zikezen", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
+           "max_positions": int(shape.get("max_position_embeddings") or 32768), "embedding": {"scale": 1.0},
+           "norm": {"eps": shape["rms_norm_eps"]}, "token_side": {"dim": 64}, "logit_softcap": 30.0,
+           "layers": [{"type": "parallel", "mixer": mixer, "mlp": moe if i % 2 else dense} for i in range(count)]}
+    if looped:
+        out["loop"] = {"start": 1, "stop": 3, "times": 2}
+    return out
+
+
 def design_run(args, shape: dict) -> int:
-    """`--design danonex|ritalorn|dagavik`: decode steps (batch 1, 8, 64 at the context asked for) and prefills of
+    """`--design danonex|ritalorn|dagavik|zikezen`: decode steps (batch 1, 8, 64 at the context asked for) and prefills of
     2,048 and 8,192 tokens of a model of that design with the shape's layer sizes, and beside each the same
-    measurement of the Qwen2.5 shape (and, for ritalorn and dagavik, of the Danonex shape) with the same number of
-    layers.  One JSON line."""
+    measurement of the Qwen2.5 shape (and, for ritalorn and dagavik, of the Danonex shape; for zikezen, of the Dagavik
+    shape) with the same number of layers (for zikezen: of layer runs).  One JSON line."""
     import torch
 
     layers = args.layers or 8
@@ -151,7 +179,11 @@ def design_run(args, shape: dict) -> int:
                         f"prefill tok/s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "context": args.ctx,
               "data": "synthetic: seeded uniform token ids, random weights N(0, 0.02)", "designs": {}}
-    if args.design == "dagavik":
+    if args.design == "zikezen":
+        configs = {"zikezen": zikezen_shape(shape, layers)}
+        if not args.alone:
+            configs.update({"dagavik": dagavik_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)})
+    elif args.design == "dagavik":
         configs = {"dagavik": dagavik_shape(shape, layers)}
         if not args.alone:
             configs.update({"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)})
@@ -409,11 +441,12 @@ def main() -> int:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
-    parser.add_argument("--design", choices=("qwen2", "danonex", "ritalorn", "dagavik"), default="qwen2",
-                        help="danonex, ritalorn, dagavik: a model of that design with the shape's layer sizes (8 layers unless "
-                             "--layers says otherwise) beside the Qwen2.5 shape (ritalorn, dagavik: and the Danonex shape) with "
-                             "as many layers: decode at batch 1, 8, 64 and prefills of 2,048 and 8,192 tokens")
-    parser.add_argument("--alone", action="store_true", help="with --design ritalorn or dagavik: that design only (for profiles)")
+    parser.add_argument("--design", choices=("qwen2", "danonex", "ritalorn", "dagavik", "zikezen"), default="qwen2",
+                        help="danonex, ritalorn, dagavik, zikezen: a model of that design with the shape's layer sizes (8 layers "
+                             "unless --layers says otherwise) beside the Qwen2.5 shape (ritalorn, dagavik: and the Danonex shape; "
+                             "zikezen: and the Dagavik shape) with as many layers: decode at batch 1, 8, 64 and prefills of 2,048 "
+                             "and 8,192 tokens")
+    parser.add_argument("--alone", action="store_true", help="with --design ritalorn, dagavik or zikezen: that design only (for profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (run with --gpus 1)")
@@ -424,7 +457,7 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
     shape = QWEN25_1P5B if args.model == "1.5b" else OTHER_SHAPES[args.model]
-    if args.design in ("danonex", "ritalorn", "dagavik"):
+    if args.design in ("danonex", "ritalorn", "dagavik", "zikezen"):
         try:
             return design_run(args, shape)
         except (Refused, Unresolved) as err:

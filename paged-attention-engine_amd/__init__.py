@@ -1,4 +1,4 @@
-"""An inference engine for the Qwen2.5 dense decoder and the Danonex and Ritalorn designs on one AMD MI355X (gfx950)."""
+"""An inference engine for the Qwen2.5 dense decoder and the Danonex, Ritalorn, Dagavik and Zikezen designs on one AMD MI355X (gfx950)."""
 
 from . import models  # noqa: F401  registers the architectures
 from . import parts   # noqa: F401  registers the built-in parts

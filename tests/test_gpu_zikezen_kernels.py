@@ -104,7 +104,7 @@ def test_terms_join_through_the_norm_after_and_the_next_reader_gets_its_form(dty
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", [dict(H=4, G=2, D=16, V=24, rot=8, bs=8), dict(H=6, G=3, D=64, V=32, rot=32, bs=16),
+@pytest.mark.parametrize("case", [dict(H=4, G=2, D=16, V=24, rot=8, bs=8), dict(H=6, G=2, D=64, V=16, rot=48, bs=16),
                                   dict(H=3, G=3, D=22, V=22, rot=10, bs=16), dict(H=5, G=1, D=18, V=10, rot=0, bs=8),
                                   dict(H=2, G=2, D=32, V=32, rot=32, bs=16)])
 def test_every_head_normed_by_itself_then_rotated_and_stored(dtype, case):
@@ -199,7 +199,7 @@ def plain_heads(q, k, v, H, G, scale, W, dtype):
 
 CASES = [dict(H=4, G=2, D=16, V=24, window=11, bs=8), dict(H=8, G=2, D=64, V=64, window=32, bs=16),
          dict(H=2, G=2, D=32, V=32, window=16, bs=16), dict(H=3, G=1, D=48, V=80, window=37, bs=16),
-         dict(H=6, G=3, D=64, V=32, window=72, bs=16)]
+         dict(H=10, G=5, D=64, V=48, window=70, bs=16)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
