@@ -152,10 +152,6 @@ int pae_embedding_positions(int dtype, float* out, const void* table, const int*
                             const int* positions, int num_tokens, int hidden, int vocab, float scale, hipStream_t stream);
 int pae_token_gate(int dtype, void* out, const void* gate, int64_t gate_stride, const void* columns, const int* ids,
                    int num_tokens, int dim, int kind, hipStream_t stream);
-int pae_token_side_rows(int dtype, float* residual, const void* rows, int64_t row_stride, const void* gate_w,
-                        const void* columns, const int* ids, const void* proj_w, int kind, const void* w_out,
-                        int w_out_is_f32, float eps, const void* w_next, int w_next_is_f32, float eps_next, void* normed,
-                        int num_rows, int hidden, int dim, hipStream_t stream);
 // float32 sums of a few output features from rows of either type: see moe.hip
 int pae_project_f32(int dtype, float* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* bias,
                     int b_is_f32, int M, int N, int K, hipStream_t stream);

@@ -100,7 +100,6 @@ def _declare(lib) -> None:
         "pae_linear_attention_step": [I, P, L, P, L, P, I, F, P, L, I, I, I, P, P, I, I, I, P, L, P, I, F, P, P, P],
         "pae_embedding_positions": [I, P, P, P, P, P, I, I, I, F, P],
         "pae_token_gate": [I, P, P, L, P, P, I, I, I, P],
-        "pae_token_side_rows": [I, P, P, L, P, P, P, P, I, P, I, F, P, I, F, P, I, I, I, P],
         "pae_moe_gate_up": [I, P, P, L, P, P, P, I, I, I, I, I, P],
         "pae_moe_down": [I, P, P, P, P, P, I, I, I, I, P],
         "pae_moe_tile_rows": [I],
@@ -233,38 +232,6 @@ def token_gate(gate: torch.Tensor, columns: torch.Tensor, ids: torch.Tensor, kin
     _check(library().pae_token_gate(code_of(gate.dtype), out.data_ptr(), gate.data_ptr(), gate.stride(0), columns.data_ptr(),
                                     ids.data_ptr(), T, dim, ACTIVATIONS[kind], _stream()))
     return out
-
-
-TOKEN_SIDE_MAX_ROWS = 64  # up to this many rows a layer's token input runs as one launch, a workgroup a row
-
-
-def token_side_rows(residual: torch.Tensor, rows: torch.Tensor, gate_w: torch.Tensor, columns: torch.Tensor,
-                    ids: torch.Tensor, proj_w: torch.Tensor, kind: str, w_out: torch.Tensor, eps: float,
-                    w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0,
-                    normed: Optional[torch.Tensor] = None) -> None:
-    """A layer's token input in one launch, for steps of a few rows: with x = `rows` [T, H] (the stream in the
-    activation type), g = act(gate_w x) * columns[ids] (rounded as the separate products round), y = proj_w g,
-    residual += y / sqrt(mean(y^2) + eps) * w_out in float32, and `normed` (optional) = the new residual normed with
-    `w_next` and `eps_next`.  `gate_w` [dim, H], `columns` [vocab, dim], `proj_w` [H, dim] in rows' type."""
-    _not_while_recording("token_side_rows")
-    _gpu(residual, rows, gate_w, columns, ids, proj_w, w_out, w_next, normed)
-    T, H = residual.shape
-    dim = gate_w.shape[0]
-    assert residual.dtype == torch.float32 and residual.is_contiguous() and kind in ACTIVATIONS
-    assert rows.shape == (T, H) and rows.stride(1) == 1
-    for w, shape in ((gate_w, (dim, H)), (proj_w, (H, dim))):
-        assert tuple(w.shape) == shape and w.is_contiguous() and w.dtype == rows.dtype
-    assert columns.dim() == 2 and columns.shape[1] == dim and columns.is_contiguous() and columns.dtype == rows.dtype
-    assert ids.dtype == torch.int32 and ids.numel() == T and ids.is_contiguous()
-    assert w_out.numel() == H and (normed is None or (w_next is not None and w_next.numel() == H))
-    if normed is not None:
-        assert normed.shape == (T, H) and normed.is_contiguous() and normed.dtype == rows.dtype
-    po, fo = _param(w_out)
-    pn, fn = _param(w_next)
-    _check(library().pae_token_side_rows(code_of(rows.dtype), residual.data_ptr(), rows.data_ptr(), rows.stride(0),
-                                         gate_w.data_ptr(), columns.data_ptr(), ids.data_ptr(), proj_w.data_ptr(),
-                                         ACTIVATIONS[kind], po, fo, float(eps), pn, fn, float(eps_next), _ptr(normed), T, H,
-                                         dim, _stream()))
 
 
 def logits_finish(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> None:

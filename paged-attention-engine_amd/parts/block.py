@@ -420,9 +420,7 @@ class SandwichBlock:
             y = self.feed_forward.forward(ctx, x)
             out = self.feed_forward_out_norm
             x, rows = self._join(stream, y, out.weight, out.spec.eps, None if has_side else follows, want_rows=has_side)
-        if has_side and self.side.joins_rows(rows.shape[0]):
-            x = self.side.join_rows(ctx, stream.residual, rows, follows)
-        elif has_side:
+        if has_side:
             y = self.side.forward(ctx, rows)
             x, _ = self._join(stream, y, self.side.weight, self.side.eps, follows)
         if follows is not None:

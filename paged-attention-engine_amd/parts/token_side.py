@@ -5,8 +5,7 @@ the layer's share of a table [vocab, table_width] that all layers declare under 
 
     g = act(W_gate x) * e;    y = W_proj g;    x <- x + y / sqrt(mean(y^2) + eps) * w
 
-The part computes y; the block adds it through the norm (`weight`, `eps`) like any sublayer's output.  In steps of a
-few rows `join_rows` does all of it, the join included, in one launch (a workgroup a row).  The
+The part computes y; the block adds it through the norm (`weight`, `eps`) like any sublayer's output.  The
 activation and the product with e are float32 and rounded once.  At bind time the layer's columns are cut out of
 the table and, like the two narrow matrices, padded with zeros to a multiple of eight (the few-row products want
 rows of 16-byte multiples; a column of zeros adds nothing).
@@ -61,21 +60,6 @@ class TokenSide(Part):
         self.gate = Linear(self.matrix(widened(weights[prefix + s.gate_name + s.weight_suffix], 0)))
         self.proj = Linear(self.matrix(widened(weights[prefix + s.proj_name + s.weight_suffix], 1)))
         self.weight = self.vector(weights[prefix + s.norm_name])
-
-    def joins_rows(self, num_rows: int) -> bool:
-        """Whether a step of `num_rows` rows takes the one-launch path."""
-        return 0 < num_rows <= K.TOKEN_SIDE_MAX_ROWS and (self.hidden_size + self.padded) * 4 <= 60 * 1024
-
-    def join_rows(self, ctx, residual: torch.Tensor, rows: torch.Tensor, next_norm=None):
-        """x <- x + norm(y) on `residual` in place, from `rows` (the stream in the activation type); returns the new
-        stream normed by `next_norm` (an RMS norm part) if one is given."""
-        if ctx.token_ids is None:
-            raise ValueError("a layer that reads a second token table needs the step's token ids")
-        normed = torch.empty(rows.shape, dtype=rows.dtype, device=rows.device) if next_norm is not None else None
-        K.token_side_rows(residual, rows, self.gate.weight, self.columns, ctx.token_ids, self.proj.weight, self.spec.activation,
-                          self.weight, self.eps, next_norm.weight if next_norm is not None else None,
-                          next_norm.spec.eps if next_norm is not None else 0.0, normed)
-        return normed
 
     def forward(self, ctx, rows: torch.Tensor):
         """`rows`: the stream in the activation type.  Returns y, as a branch's last product returns it."""

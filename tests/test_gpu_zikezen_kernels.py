@@ -63,37 +63,6 @@ def test_the_tokens_columns_gate_a_narrow_product(dtype, dim):
     close(got, want, 1e-6 if dtype == torch.float32 else 5e-3, f"token gate {dim}")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(64, 8), (90, 8), (192, 24), (1536, 64)])
-def test_a_layers_token_input_in_one_launch(dtype, shape):
-    """Gate product, activation, the token's columns, second product, norm and join for a few rows at once, against the
-    plain functions with the separate products' roundings; then the next reader's norm."""
-    H, dim = shape
-    gen = torch.Generator().manual_seed(H + dim)
-    T, eps, eps_next = 9, 1e-5, 2e-6
-    res = torch.randn((T, H), generator=gen) * 3.0
-    gate_w = (torch.randn((dim, H), generator=gen) * H ** -0.5).to(dtype)
-    proj_w = (torch.randn((H, dim), generator=gen) * 0.3).to(dtype)
-    columns = torch.randn((40, dim), generator=gen).to(dtype)
-    ids = torch.randint(0, 40, (T,), generator=gen, dtype=torch.int32)
-    w_out = 1.0 + 0.2 * torch.randn((H,), generator=gen)
-    w_next = 1.0 + 0.2 * torch.randn((H,), generator=gen)
-    rows = res.to(dtype)
-    plain.STORAGE = dtype
-    try:
-        g = plain.stored(plain.gelu_tanh(plain.product(rows.double(), gate_w.double())) * columns.double()[ids.long()])
-    finally:
-        plain.STORAGE = None
-    want = res.double() + plain.rms_norm(g @ proj_w.double().T, w_out.double(), eps)
-    got = res.to(DEV)
-    normed = torch.empty((T, H), dtype=dtype, device=DEV)
-    K().token_side_rows(got, rows.to(DEV), gate_w.to(DEV), columns.to(DEV), ids.to(DEV), proj_w.to(DEV), "gelu_tanh",
-                        w_out.to(DEV), eps, w_next.to(DEV), eps_next, normed)
-    rel = 2e-6 if dtype == torch.float32 else 4e-3  # (a gate sum next to a rounding border may round the other way)
-    close(got, want, rel, f"stream {shape}")
-    close(normed, plain.rms_norm(want, w_next.double(), eps_next), max(rel, 5e-3 if dtype == torch.bfloat16 else rel), f"next norm {shape}")
-
-
 # ----------------------------------------------------------------------------- a sublayer's output joins through its norm
 
 
