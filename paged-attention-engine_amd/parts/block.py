@@ -401,15 +401,21 @@ class SandwichBlock:
                     next_norm.spec.eps if next_norm is not None else 0.0, normed, rows)
         return normed, rows
 
+    def _next_first_norm(self, stream: ResidualStream):
+        """The first norm of the block that follows, if that block takes its rows prepared (the model says so) and
+        the norm is one the joining kernel can form (an RMS norm with a plain weight); else None."""
+        norm = stream.next_norm if stream.prepared_wanted_next else None
+        if norm is None or not isinstance(norm, type(self.mixer_norm)) or norm.spec.weight_offset:
+            return None
+        return norm
+
     def forward(self, ctx, stream: ResidualStream) -> None:
         if stream.pending is not None or stream.owed is not None or stream.copies != 1:
             raise ValueError("a block with norms around its sublayers follows one that left the stream in another form")
         ctx.sink = None
         prepared, stream.prepared = stream.prepared, None
         x = prepared[1] if prepared is not None and prepared[0] is self.mixer_norm else self.mixer_norm.forward(stream)
-        # what follows the layer's last sublayer: the next block's first norm, if that block takes prepared rows
-        follows = stream.next_norm if stream.prepared_wanted_next and isinstance(stream.next_norm, type(self.mixer_norm)) \
-            and not stream.next_norm.spec.weight_offset else None
+        follows = self._next_first_norm(stream)
         has_ff, has_side = self.feed_forward is not None, self.side is not None
         y = self.mixer.forward(ctx, x)
         out = self.mixer_out_norm

@@ -168,6 +168,18 @@ def test_a_layer_that_runs_twice_is_one_set_of_tensors():
     assert sum(1 for name in shapes if name.startswith("l0.norm1")) == 2  # norm1 and norm1b, once each
 
 
+def test_the_bench_shape_is_a_config_the_reader_takes():
+    """`bench.py --design zikezen` builds its model from a config of its own making: as many layer runs as asked for."""
+    import bench
+
+    for runs in (2, 8):
+        plan = pae.read_config_dict(bench.zikezen_shape(bench.QWEN25_1P5B, runs)).plan()
+        assert len(plan.schedule) == runs and plan.hidden_size == 1536
+    plan = pae.read_config_dict(bench.zikezen_shape(bench.QWEN25_1P5B, 8)).plan()
+    assert [e.layer for e in plan.schedule] == [0, 1, 2, 1, 2, 3, 4, 5] and [e.add_embedding for e in plan.schedule].count(True) == 1
+    assert {type(layer.feed_forward).__name__ for layer in plan.layers} == {"FeedForwardSpec", "ExpertsSpec"}
+
+
 # ----------------------------------------------------------------------------- the plain implementation, pinned
 
 
